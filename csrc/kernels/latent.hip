@@ -1,0 +1,502 @@
+// Kernels of decoders with a 32-bit residual stream, latent (low-rank, shared-key) attention and
+// group-limited sigmoid routing, for gfx950.  Every kernel exists for bf16 and for fp32 activations
+// (dtype 0 / 1 in the entry points); what a design computes in 32-bit (norms, angles, scores,
+// softmax, routing, the residual sum) is fp32 in both.
+//
+//   embed_scale        residual[t] = embed[id[t]] * scale                                (fp32 out)
+//   add_rmsnorm        residual += delta;  y = residual * rsqrt(mean(residual^2) + eps) * w
+//   rmsnorm_rows       y = x * rsqrt(mean(x^2) + eps) * w over a column range of a wider row
+//   latent_kv_write    a token's compressed KV entry: RMS-normed latent | rotated shared key part
+//                      -> paged cache row [rank + rot]
+//   rope_pairs         interleaved-pair rotary embedding of a column range of every head, in place
+//   latent_attention   causal attention of query rows in latent space over the paged entries with an
+//                      optional per-head sink logit in the softmax denominator
+//   sigmoid_gate       y[t, h, :] *= sigmoid(g[t, h])
+//   relu_sq            y = relu(x)^2
+//   glu_clamp          y = g' * sigmoid(alpha g') * (u' + bias),  g' = min(g, limit), u' = clamp(u, +-limit)
+//   group_topk         sigmoid scores -> best groups by the sum of their two largest -> top-k experts
+//   gather_rows        xs[r] = x[idx[r]]
+//   moe_finish         residual[t] += sum_k w[t,k] * y[pos[t,k]] + gate[t] * shared[t]
+//
+// Sizes are free (no multiple-of-8 requirements): these are the plain kernels every shape can take.
+#include "common.h"
+
+namespace {
+
+template <typename T> struct Conv;
+template <> struct Conv<float> {
+  static __device__ __forceinline__ float ld(const float* p) { return *p; }
+  static __device__ __forceinline__ void st(float* p, float v) { *p = v; }
+};
+template <> struct Conv<bf16_t> {
+  static __device__ __forceinline__ float ld(const bf16_t* p) { return (float)*p; }
+  static __device__ __forceinline__ void st(bf16_t* p, float v) { *p = (bf16_t)v; }
+};
+
+__device__ __forceinline__ float block_sum(float v, float* red) {
+  v = wave_reduce_sum(v);
+  const int tid = threadIdx.x;
+  __syncthreads();
+  if ((tid & 63) == 0) red[tid >> 6] = v;
+  __syncthreads();
+  float s = 0.f;
+  for (int i = 0; i < (int)(blockDim.x >> 6); ++i) s += red[i];
+  return s;
+}
+
+__device__ __forceinline__ float block_max(float v, float* red) {
+  v = wave_reduce_max(v);
+  const int tid = threadIdx.x;
+  __syncthreads();
+  if ((tid & 63) == 0) red[tid >> 6] = v;
+  __syncthreads();
+  float s = red[0];
+  for (int i = 1; i < (int)(blockDim.x >> 6); ++i) s = fmaxf(s, red[i]);
+  return s;
+}
+
+__device__ __forceinline__ float sigmoidf(float x) { return 1.f / (1.f + expf(-x)); }
+
+// ---------------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void embed_scale_kernel(const long* __restrict__ ids, const T* __restrict__ embed,
+                                                          float* __restrict__ out, int width, float scale) {
+  const long row = blockIdx.x;
+  const T* e = embed + ids[row] * (long)width;
+  float* o = out + row * width;
+  for (int i = threadIdx.x; i < width; i += 256) o[i] = Conv<T>::ld(e + i) * scale;
+}
+
+// residual fp32 [rows, n] (+= delta, row stride d_stride) -> y (row stride y_stride)
+template <typename T>
+__global__ __launch_bounds__(256) void add_rmsnorm_kernel(float* __restrict__ residual, const T* __restrict__ delta,
+                                                          long d_stride, const float* __restrict__ w,
+                                                          T* __restrict__ y, long y_stride, int n, float eps) {
+  __shared__ float red[4];
+  const long row = blockIdx.x;
+  float* r = residual + row * n;
+  float ss = 0.f;
+  if (delta) {
+    const T* d = delta + row * d_stride;
+    for (int i = threadIdx.x; i < n; i += 256) {
+      const float v = r[i] + Conv<T>::ld(d + i);
+      r[i] = v;  // read back below by the same thread
+      ss += v * v;
+    }
+  } else {
+    for (int i = threadIdx.x; i < n; i += 256) {
+      const float v = r[i];
+      ss += v * v;
+    }
+  }
+  const float inv = 1.f / sqrtf(block_sum(ss, red) / (float)n + eps);
+  if (!y) return;
+  T* yr = y + row * y_stride;
+  for (int i = threadIdx.x; i < n; i += 256) Conv<T>::st(yr + i, r[i] * inv * w[i]);
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void rmsnorm_rows_kernel(const T* __restrict__ x, long x_stride,
+                                                           const float* __restrict__ w, T* __restrict__ y,
+                                                           long y_stride, int n, float eps) {
+  __shared__ float red[4];
+  const long row = blockIdx.x;
+  const T* xr = x + row * x_stride;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < n; i += 256) {
+    const float v = Conv<T>::ld(xr + i);
+    ss += v * v;
+  }
+  const float inv = 1.f / sqrtf(block_sum(ss, red) / (float)n + eps);
+  T* yr = y + row * y_stride;
+  for (int i = threadIdx.x; i < n; i += 256) Conv<T>::st(yr + i, Conv<T>::ld(xr + i) * inv * w[i]);
+}
+
+// x [rows, >= rank + rot] (row stride x_stride): columns [0, rank) are RMS-normed with w, columns
+// [rank, rank + rot) are the shared key part, whose first rot_dims columns rotate in interleaved
+// pairs (2i, 2i+1) by the angle table cos_sin[pos] = cos[0 .. rot_dims/2) | sin[0 .. rot_dims/2).
+// The entry goes to cache + (slot / 64) * page_stride + (slot % 64) * (rank + rot); slot < 0 skips.
+template <typename T>
+__global__ __launch_bounds__(256) void latent_kv_write_kernel(const T* __restrict__ x, long x_stride,
+                                                              const float* __restrict__ w,
+                                                              const int* __restrict__ positions,
+                                                              const long* __restrict__ slots,
+                                                              const float* __restrict__ cos_sin, T* __restrict__ cache,
+                                                              long page_stride, int rank, int rot, int rot_dims,
+                                                              float eps) {
+  __shared__ float red[4];
+  const long row = blockIdx.x;
+  const long slot = slots[row];
+  if (slot < 0) return;
+  const T* xr = x + row * x_stride;
+  T* dst = cache + (slot / PAGE) * page_stride + (slot % PAGE) * (long)(rank + rot);
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < rank; i += 256) {
+    const float v = Conv<T>::ld(xr + i);
+    ss += v * v;
+  }
+  const float inv = 1.f / sqrtf(block_sum(ss, red) / (float)rank + eps);
+  for (int i = threadIdx.x; i < rank; i += 256) Conv<T>::st(dst + i, Conv<T>::ld(xr + i) * inv * w[i]);
+  const int half = rot_dims >> 1;
+  const float* cs = cos_sin + (long)positions[row] * rot_dims;
+  for (int i = threadIdx.x; i < half; i += 256) {
+    const float u = Conv<T>::ld(xr + rank + 2 * i), v = Conv<T>::ld(xr + rank + 2 * i + 1);
+    const float c = cs[i], s = cs[half + i];
+    Conv<T>::st(dst + rank + 2 * i, u * c - v * s);
+    Conv<T>::st(dst + rank + 2 * i + 1, v * c + u * s);
+  }
+  for (int i = rot_dims + threadIdx.x; i < rot; i += 256) dst[rank + i] = xr[rank + i];
+}
+
+// q [rows, heads, head_stride]: columns [col0, col0 + rot_dims) of every head rotate in place
+template <typename T>
+__global__ __launch_bounds__(256) void rope_pairs_kernel(T* __restrict__ q, long row_stride, long head_stride,
+                                                         const int* __restrict__ positions,
+                                                         const float* __restrict__ cos_sin, int heads, int col0,
+                                                         int rot_dims) {
+  const long row = blockIdx.x;
+  const int half = rot_dims >> 1;
+  const float* cs = cos_sin + (long)positions[row] * rot_dims;
+  for (int i = threadIdx.x; i < heads * half; i += 256) {
+    const int h = i / half, j = i % half;
+    T* p = q + row * row_stride + h * head_stride + col0 + 2 * j;
+    const float u = Conv<T>::ld(p), v = Conv<T>::ld(p + 1);
+    const float c = cs[j], s = cs[half + j];
+    Conv<T>::st(p, u * c - v * s);
+    Conv<T>::st(p + 1, v * c + u * s);
+  }
+}
+
+// ---------------------------------------------------------------------------------
+// Latent attention, plain form.  One 256-thread workgroup per (query row, head).  The query is
+// q_lat [rank] (the head's unrotated query carried into latent space) | q_rot [rot]; key j of the
+// row's sequence is the cache entry [rank + rot] and its value the entry's first rank columns.
+//   score_j = (q_lat . c_j + q_rot . r_j) * scale,   j <= position
+//   out     = sum_j exp(score_j - m) c_j / (sum_j exp(score_j - m) + exp(sink - m))
+// Keys are taken 256 at a time (a thread scores one key, then owns output columns tid, tid+256, ..).
+// ---------------------------------------------------------------------------------
+#define LAT_MAX_COLS 8  // rank <= 2048
+
+template <typename T>
+__global__ __launch_bounds__(256) void latent_attention_kernel(
+    const T* __restrict__ q_lat, long ql_row, long ql_head, const T* __restrict__ q_rot, long qr_row, long qr_head,
+    const T* __restrict__ cache, long page_stride, const int* __restrict__ block_tables, int bt_stride,
+    const int* __restrict__ row_seq, const int* __restrict__ positions, const float* __restrict__ sink,
+    T* __restrict__ out, long o_row, long o_head, int rank, int rot, float scale) {
+  extern __shared__ float smem[];
+  float* qs = smem;             // [rank + rot], pre-scaled
+  float* ps = smem + rank + rot;  // [256]
+  __shared__ float red[4];
+  const int row = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
+  const int width = rank + rot;
+  const int ctx = positions[row] + 1;
+  const int seq = row_seq ? row_seq[row] : row;
+  const int* bt = block_tables + (long)seq * bt_stride;
+  for (int i = tid; i < rank; i += 256) qs[i] = Conv<T>::ld(q_lat + row * ql_row + h * ql_head + i) * scale;
+  for (int i = tid; i < rot; i += 256) qs[rank + i] = Conv<T>::ld(q_rot + row * qr_row + h * qr_head + i) * scale;
+  float m = sink ? sink[h] : -INFINITY;
+  float l = sink ? 1.f : 0.f;
+  float acc[LAT_MAX_COLS];
+#pragma unroll
+  for (int c = 0; c < LAT_MAX_COLS; ++c) acc[c] = 0.f;
+  __syncthreads();
+  for (int j0 = 0; j0 < ctx; j0 += 256) {
+    const int j = j0 + tid;
+    float s = -INFINITY;
+    if (j < ctx) {
+      const T* k = cache + (long)bt[j / PAGE] * page_stride + (long)(j % PAGE) * width;
+      float a = 0.f;
+      for (int d = 0; d < width; ++d) a += qs[d] * Conv<T>::ld(k + d);
+      s = a;
+    }
+    const float mc = block_max(s, red);
+    const float mn = fmaxf(m, mc);
+    const float p = j < ctx ? expf(s - mn) : 0.f;
+    const float corr = (m == -INFINITY) ? 0.f : expf(m - mn);
+    ps[tid] = p;
+    const float psum = block_sum(p, red);  // (its barriers also publish ps)
+    l = l * corr + psum;
+    m = mn;
+    const int nk = min(256, ctx - j0);
+#pragma unroll
+    for (int c = 0; c < LAT_MAX_COLS; ++c) {
+      const int d = c * 256 + tid;
+      if (d < rank) {
+        float a = acc[c] * corr;
+        for (int jj = 0; jj < nk; ++jj) {
+          const int key = j0 + jj;
+          a += ps[jj] * Conv<T>::ld(cache + (long)bt[key / PAGE] * page_stride + (long)(key % PAGE) * width + d);
+        }
+        acc[c] = a;
+      }
+    }
+    __syncthreads();  // ps is rewritten by the next round
+  }
+  const float inv = l > 0.f ? 1.f / l : 0.f;
+#pragma unroll
+  for (int c = 0; c < LAT_MAX_COLS; ++c) {
+    const int d = c * 256 + tid;
+    if (d < rank) Conv<T>::st(out + row * o_row + h * o_head + d, acc[c] * inv);
+  }
+}
+
+// y [rows, heads, vdim] (contiguous) *= sigmoid(g[row * g_stride + head])
+template <typename T>
+__global__ __launch_bounds__(256) void sigmoid_gate_kernel(T* __restrict__ y, const T* __restrict__ g, long g_stride,
+                                                           int heads, int vdim) {
+  const long row = blockIdx.x;
+  T* yr = y + row * heads * vdim;
+  for (int i = threadIdx.x; i < heads * vdim; i += 256) {
+    const float s = sigmoidf(Conv<T>::ld(g + row * g_stride + i / vdim));
+    Conv<T>::st(yr + i, Conv<T>::ld(yr + i) * s);
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void relu_sq_kernel(const T* __restrict__ x, T* __restrict__ y, long n) {
+  for (long i = blockIdx.x * 256L + threadIdx.x; i < n; i += (long)gridDim.x * 256) {
+    const float v = fmaxf(Conv<T>::ld(x + i), 0.f);
+    Conv<T>::st(y + i, v * v);
+  }
+}
+
+// x [rows, 2 * inter] (row stride x_stride): gate columns then up columns -> y [rows, inter]
+template <typename T>
+__global__ __launch_bounds__(256) void glu_clamp_kernel(const T* __restrict__ x, long x_stride, T* __restrict__ y,
+                                                        int inter, long total, float limit, float alpha,
+                                                        float up_bias) {
+  for (long i = blockIdx.x * 256L + threadIdx.x; i < total; i += (long)gridDim.x * 256) {
+    const long r = i / inter;
+    const int c = (int)(i % inter);
+    const float g = fminf(Conv<T>::ld(x + r * x_stride + c), limit);
+    const float u = fminf(fmaxf(Conv<T>::ld(x + r * x_stride + inter + c), -limit), limit);
+    Conv<T>::st(y + i, g * sigmoidf(alpha * g) * (u + up_bias));
+  }
+}
+
+// ---------------------------------------------------------------------------------
+// Group-limited top-k routing on sigmoid scores.  logits fp32 [tokens, cols] (cols >= experts; with
+// `extra` column `experts` holds a per-token gate logit whose sigmoid goes to extra_out).  Experts
+// form `groups` equal runs of neighbours; a group scores the sum of its two largest scores (its
+// only one for groups of one); experts outside the `keep` best groups cannot be chosen.  Weights
+// are the chosen scores times route_scale (not renormalised).  Ties go to the lower index.
+// One wave per token.
+// ---------------------------------------------------------------------------------
+#define ROUTE_MAX_EXPERTS 1024
+
+__global__ __launch_bounds__(64) void group_topk_kernel(const float* __restrict__ logits, int cols,
+                                                        float* __restrict__ weights, int* __restrict__ ids,
+                                                        float* __restrict__ extra_out, int experts, int groups,
+                                                        int keep, int topk, float route_scale) {
+  __shared__ float s[ROUTE_MAX_EXPERTS];
+  __shared__ float gs[ROUTE_MAX_EXPERTS];
+  const long t = blockIdx.x;
+  const int lane = threadIdx.x;
+  const float* z = logits + t * cols;
+  for (int e = lane; e < experts; e += 64) s[e] = sigmoidf(z[e]);
+  if (extra_out && lane == 0) extra_out[t] = sigmoidf(z[experts]);
+  __syncthreads();
+  const int per = experts / groups;
+  for (int g = lane; g < groups; g += 64) {
+    float a = -1.f, b = -1.f;  // two largest (scores are > 0)
+    for (int e = g * per; e < (g + 1) * per; ++e) {
+      const float v = s[e];
+      if (v > a) { b = a; a = v; }
+      else if (v > b) { b = v; }
+    }
+    gs[g] = per > 1 ? a + b : a;
+  }
+  __syncthreads();
+  // the keep best groups: group g stays when fewer than keep groups beat it (a tie counts for the lower index)
+  for (int g = lane; g < groups; g += 64) {
+    int ahead = 0;
+    const float v = gs[g];
+    for (int o = 0; o < groups; ++o) ahead += (gs[o] > v) || (gs[o] == v && o < g);
+    if (ahead >= keep)
+      for (int e = g * per; e < (g + 1) * per; ++e) s[e] = -1.f;
+  }
+  __syncthreads();
+  for (int k = 0; k < topk; ++k) {
+    float best = -2.f;
+    int bi = 0x7fffffff;
+    for (int e = lane; e < experts; e += 64)
+      if (s[e] > best) { best = s[e]; bi = e; }
+    for (int off = 32; off > 0; off >>= 1) {
+      const float ob = __shfl_xor(best, off, 64);
+      const int oi = __shfl_xor(bi, off, 64);
+      if (ob > best || (ob == best && oi < bi)) { best = ob; bi = oi; }
+    }
+    if (lane == 0) {
+      weights[t * topk + k] = best * route_scale;
+      ids[t * topk + k] = bi;
+    }
+    __syncthreads();
+    if (lane == 0) s[bi] = -3.f;
+    __syncthreads();
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void gather_rows_kernel(const T* __restrict__ x, const int* __restrict__ idx,
+                                                          T* __restrict__ xs, int n) {
+  const long row = blockIdx.x;
+  const T* src = x + (long)idx[row] * n;
+  for (int i = threadIdx.x; i < n; i += 256) xs[row * n + i] = src[i];
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void moe_finish_kernel(float* __restrict__ residual, const T* __restrict__ y,
+                                                         const float* __restrict__ weights,
+                                                         const int* __restrict__ pos, int topk,
+                                                         const T* __restrict__ shared, const float* __restrict__ gate,
+                                                         int n) {
+  const long t = blockIdx.x;
+  const float sg = shared ? (gate ? gate[t] : 1.f) : 0.f;
+  for (int i = threadIdx.x; i < n; i += 256) {
+    float a = 0.f;
+    for (int k = 0; k < topk; ++k) {
+      const float w = weights[t * topk + k];
+      if (w != 0.f) a += w * Conv<T>::ld(y + (long)pos[t * topk + k] * n + i);
+    }
+    if (shared) a += sg * Conv<T>::ld(shared + t * n + i);
+    residual[t * n + i] += a;
+  }
+}
+
+inline int flat_grid(long total) {
+  long b = (total + 255) / 256;
+  return (int)(b < 1 ? 1 : (b > 65535 ? 65535 : b));
+}
+
+}  // namespace
+
+#define DISPATCH(dtype, CALL_BF16, CALL_F32) \
+  do {                                       \
+    if ((dtype) == 0) { CALL_BF16; }         \
+    else if ((dtype) == 1) { CALL_F32; }     \
+    else return -2;                          \
+  } while (0)
+
+VPSA_EXPORT int vpsa_embed_scale(const long* ids, const void* embed, float* out, int rows, int width, float scale,
+                                 int dtype, hipStream_t st) {
+  if (rows <= 0) return 0;
+  DISPATCH(dtype,
+           hipLaunchKernelGGL(embed_scale_kernel<bf16_t>, dim3(rows), dim3(256), 0, st, ids, (const bf16_t*)embed, out, width, scale),
+           hipLaunchKernelGGL(embed_scale_kernel<float>, dim3(rows), dim3(256), 0, st, ids, (const float*)embed, out, width, scale));
+  return 0;
+}
+
+VPSA_EXPORT int vpsa_add_rmsnorm(float* residual, const void* delta, long d_stride, const float* w, void* y,
+                                 long y_stride, int rows, int n, float eps, int dtype, hipStream_t st) {
+  if (rows <= 0) return 0;
+  DISPATCH(dtype,
+           hipLaunchKernelGGL(add_rmsnorm_kernel<bf16_t>, dim3(rows), dim3(256), 0, st, residual, (const bf16_t*)delta, d_stride, w, (bf16_t*)y, y_stride, n, eps),
+           hipLaunchKernelGGL(add_rmsnorm_kernel<float>, dim3(rows), dim3(256), 0, st, residual, (const float*)delta, d_stride, w, (float*)y, y_stride, n, eps));
+  return 0;
+}
+
+VPSA_EXPORT int vpsa_rmsnorm_rows(const void* x, long x_stride, const float* w, void* y, long y_stride, int rows,
+                                  int n, float eps, int dtype, hipStream_t st) {
+  if (rows <= 0) return 0;
+  DISPATCH(dtype,
+           hipLaunchKernelGGL(rmsnorm_rows_kernel<bf16_t>, dim3(rows), dim3(256), 0, st, (const bf16_t*)x, x_stride, w, (bf16_t*)y, y_stride, n, eps),
+           hipLaunchKernelGGL(rmsnorm_rows_kernel<float>, dim3(rows), dim3(256), 0, st, (const float*)x, x_stride, w, (float*)y, y_stride, n, eps));
+  return 0;
+}
+
+VPSA_EXPORT int vpsa_latent_kv_write(const void* x, long x_stride, const float* w, const int* positions,
+                                     const long* slots, const float* cos_sin, void* cache, long page_stride,
+                                     int rows, int rank, int rot, int rot_dims, float eps, int dtype,
+                                     hipStream_t st) {
+  if (rows <= 0) return 0;
+  if (rot_dims > rot || (rot_dims & 1)) return -1;
+  DISPATCH(dtype,
+           hipLaunchKernelGGL(latent_kv_write_kernel<bf16_t>, dim3(rows), dim3(256), 0, st, (const bf16_t*)x, x_stride, w, positions, slots, cos_sin, (bf16_t*)cache, page_stride, rank, rot, rot_dims, eps),
+           hipLaunchKernelGGL(latent_kv_write_kernel<float>, dim3(rows), dim3(256), 0, st, (const float*)x, x_stride, w, positions, slots, cos_sin, (float*)cache, page_stride, rank, rot, rot_dims, eps));
+  return 0;
+}
+
+VPSA_EXPORT int vpsa_rope_pairs(void* q, long row_stride, long head_stride, const int* positions,
+                                const float* cos_sin, int rows, int heads, int col0, int rot_dims, int dtype,
+                                hipStream_t st) {
+  if (rows <= 0 || rot_dims == 0) return 0;
+  if (rot_dims & 1) return -1;
+  DISPATCH(dtype,
+           hipLaunchKernelGGL(rope_pairs_kernel<bf16_t>, dim3(rows), dim3(256), 0, st, (bf16_t*)q, row_stride, head_stride, positions, cos_sin, heads, col0, rot_dims),
+           hipLaunchKernelGGL(rope_pairs_kernel<float>, dim3(rows), dim3(256), 0, st, (float*)q, row_stride, head_stride, positions, cos_sin, heads, col0, rot_dims));
+  return 0;
+}
+
+VPSA_EXPORT int vpsa_latent_attention(const void* q_lat, long ql_row, long ql_head, const void* q_rot, long qr_row,
+                                      long qr_head, const void* cache, long page_stride, const int* block_tables,
+                                      int bt_stride, const int* row_seq, const int* positions, const float* sink,
+                                      void* out, long o_row, long o_head, int rows, int heads, int rank, int rot,
+                                      float scale, int dtype, hipStream_t st) {
+  if (rows <= 0) return 0;
+  if (rank > LAT_MAX_COLS * 256 || heads > 65535) return -1;
+  const size_t lds = (size_t)(rank + rot + 256) * sizeof(float);
+  if (lds > 60 * 1024) return -1;
+  dim3 grid(rows, heads);
+  DISPATCH(dtype,
+           hipLaunchKernelGGL(latent_attention_kernel<bf16_t>, grid, dim3(256), lds, st, (const bf16_t*)q_lat, ql_row, ql_head, (const bf16_t*)q_rot, qr_row, qr_head, (const bf16_t*)cache, page_stride, block_tables, bt_stride, row_seq, positions, sink, (bf16_t*)out, o_row, o_head, rank, rot, scale),
+           hipLaunchKernelGGL(latent_attention_kernel<float>, grid, dim3(256), lds, st, (const float*)q_lat, ql_row, ql_head, (const float*)q_rot, qr_row, qr_head, (const float*)cache, page_stride, block_tables, bt_stride, row_seq, positions, sink, (float*)out, o_row, o_head, rank, rot, scale));
+  return 0;
+}
+
+VPSA_EXPORT int vpsa_sigmoid_gate(void* y, const void* g, long g_stride, int rows, int heads, int vdim, int dtype,
+                                  hipStream_t st) {
+  if (rows <= 0) return 0;
+  DISPATCH(dtype,
+           hipLaunchKernelGGL(sigmoid_gate_kernel<bf16_t>, dim3(rows), dim3(256), 0, st, (bf16_t*)y, (const bf16_t*)g, g_stride, heads, vdim),
+           hipLaunchKernelGGL(sigmoid_gate_kernel<float>, dim3(rows), dim3(256), 0, st, (float*)y, (const float*)g, g_stride, heads, vdim));
+  return 0;
+}
+
+VPSA_EXPORT int vpsa_relu_sq(const void* x, void* y, long n, int dtype, hipStream_t st) {
+  if (n <= 0) return 0;
+  DISPATCH(dtype,
+           hipLaunchKernelGGL(relu_sq_kernel<bf16_t>, dim3(flat_grid(n)), dim3(256), 0, st, (const bf16_t*)x, (bf16_t*)y, n),
+           hipLaunchKernelGGL(relu_sq_kernel<float>, dim3(flat_grid(n)), dim3(256), 0, st, (const float*)x, (float*)y, n));
+  return 0;
+}
+
+VPSA_EXPORT int vpsa_glu_clamp(const void* x, long x_stride, void* y, int rows, int inter, float limit, float alpha,
+                               float up_bias, int dtype, hipStream_t st) {
+  const long total = (long)rows * inter;
+  if (total <= 0) return 0;
+  DISPATCH(dtype,
+           hipLaunchKernelGGL(glu_clamp_kernel<bf16_t>, dim3(flat_grid(total)), dim3(256), 0, st, (const bf16_t*)x, x_stride, (bf16_t*)y, inter, total, limit, alpha, up_bias),
+           hipLaunchKernelGGL(glu_clamp_kernel<float>, dim3(flat_grid(total)), dim3(256), 0, st, (const float*)x, x_stride, (float*)y, inter, total, limit, alpha, up_bias));
+  return 0;
+}
+
+VPSA_EXPORT int vpsa_group_topk(const float* logits, int cols, float* weights, int* ids, float* extra_out,
+                                int tokens, int experts, int groups, int keep, int topk, float route_scale,
+                                hipStream_t st) {
+  if (tokens <= 0) return 0;
+  if (experts > ROUTE_MAX_EXPERTS || groups < 1 || experts % groups || keep < 1 || keep > groups ||
+      topk > experts / groups * keep || cols < experts + (extra_out ? 1 : 0))
+    return -1;
+  hipLaunchKernelGGL(group_topk_kernel, dim3(tokens), dim3(64), 0, st, logits, cols, weights, ids, extra_out,
+                     experts, groups, keep, topk, route_scale);
+  return 0;
+}
+
+VPSA_EXPORT int vpsa_gather_rows(const void* x, const int* idx, void* xs, int rows, int n, int dtype,
+                                 hipStream_t st) {
+  if (rows <= 0) return 0;
+  DISPATCH(dtype,
+           hipLaunchKernelGGL(gather_rows_kernel<bf16_t>, dim3(rows), dim3(256), 0, st, (const bf16_t*)x, idx, (bf16_t*)xs, n),
+           hipLaunchKernelGGL(gather_rows_kernel<float>, dim3(rows), dim3(256), 0, st, (const float*)x, idx, (float*)xs, n));
+  return 0;
+}
+
+VPSA_EXPORT int vpsa_moe_finish(float* residual, const void* y, const float* weights, const int* pos, int topk,
+                                const void* shared, const float* gate, int tokens, int n, int dtype,
+                                hipStream_t st) {
+  if (tokens <= 0) return 0;
+  DISPATCH(dtype,
+           hipLaunchKernelGGL(moe_finish_kernel<bf16_t>, dim3(tokens), dim3(256), 0, st, residual, (const bf16_t*)y, weights, pos, topk, (const bf16_t*)shared, gate, n),
+           hipLaunchKernelGGL(moe_finish_kernel<float>, dim3(tokens), dim3(256), 0, st, residual, (const float*)y, weights, pos, topk, (const float*)shared, gate, n));
+  return 0;
+}

@@ -9,7 +9,8 @@
 // expert's contiguous row range.
 #include "common.h"
 
-#define MAX_EXPERTS 64
+#define MAX_EXPERTS 64        // top-k softmax keeps a token's scores in registers
+#define ALIGN_MAX_EXPERTS 1024  // the counting sort keeps its counters in LDS
 #define MAX_TOPK 8
 
 __global__ __launch_bounds__(256) void moe_topk_softmax_kernel(const uint16_t* __restrict__ logits,
@@ -57,10 +58,10 @@ __global__ __launch_bounds__(1024) void moe_align_kernel(const int* __restrict__
                                                          int* __restrict__ pos,
                                                          int* __restrict__ sorted_tok, int n_pairs,
                                                          int n_experts, int topk) {
-  __shared__ int cnt[MAX_EXPERTS + 1];
-  __shared__ int base[MAX_EXPERTS + 1];
+  __shared__ int cnt[ALIGN_MAX_EXPERTS + 1];
+  __shared__ int base[ALIGN_MAX_EXPERTS + 1];
   const int tid = threadIdx.x;
-  if (tid <= n_experts) cnt[tid] = 0;
+  for (int e = tid; e <= n_experts; e += 1024) cnt[e] = 0;
   __syncthreads();
   for (int i = tid; i < n_pairs; i += 1024) atomicAdd(&cnt[ids[i]], 1);
   __syncthreads();
@@ -139,7 +140,7 @@ VPSA_EXPORT int vpsa_moe_topk_softmax(const void* logits, float* weights, int* i
 
 VPSA_EXPORT int vpsa_moe_align(const int* ids, int* offsets, int* pos, int* sorted_tok,
                                int n_pairs, int n_experts, int topk, hipStream_t stream) {
-  if (n_experts > MAX_EXPERTS) return -1;
+  if (n_experts > ALIGN_MAX_EXPERTS) return -1;
   hipLaunchKernelGGL(moe_align_kernel, dim3(1), dim3(1024), 0, stream, ids, offsets, pos,
                      sorted_tok, n_pairs, n_experts, topk);
   return 0;

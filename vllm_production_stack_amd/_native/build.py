@@ -22,6 +22,8 @@ CSRC = ROOT / "csrc"
 ROCM = Path(os.environ.get("ROCM_PATH", "/opt/rocm"))
 
 HIPCC = shutil.which("hipcc") or str(ROCM / "bin" / "hipcc")
+# every device compile: ordinary float code must not be turned into packed fp32 instructions
+HIP_FLAGS = ["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 CXX = shutil.which("g++") or "g++"
 
 # target name -> (compiler kind, sources relative to csrc/, extra flags)
@@ -31,7 +33,7 @@ TARGETS = {
         ["kernels/elementwise.hip", "kernels/attention.hip", "kernels/kvcache.hip", "kernels/moe.hip",
          "kernels/lora.hip", "kernels/gemm.hip", "kernels/rans.hip", "kernels/sampling.hip",
          "kernels/grouped_gemm.hip", "kernels/packed_gemm.hip", "kernels/dense_attention.hip",
-         "kernels/tile_gemm.hip"],
+         "kernels/tile_gemm.hip", "kernels/latent.hip"],
         [],
     ),
     "vpsa_kvio": ("hip", ["kvio/kvio.cpp"], []),
@@ -97,12 +99,12 @@ def build_target(name: str, force: bool = False) -> Path | None:
             obj = objdir / (path.stem + ".o")
             if force or _stale(obj, [path]):
                 _run([HIPCC, "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden",
-                      "-I", str(CSRC), *SOURCE_FLAGS.get(src, []), "-c", str(path), "-o", str(obj)])
+                      *HIP_FLAGS, "-I", str(CSRC), *SOURCE_FLAGS.get(src, []), "-c", str(path), "-o", str(obj)])
             objs.append(str(obj))
         cmd = [HIPCC, "--offload-arch=gfx950", *shared, *objs, "-o", str(out), *flags]
     elif kind == "hip":
         cmd = [HIPCC, "--offload-arch=gfx950", "-O3", "-std=c++17", *shared,
-               "-fvisibility=hidden", "-I", str(CSRC), *map(str, paths), "-o", str(out), *flags]
+               "-fvisibility=hidden", *HIP_FLAGS, "-I", str(CSRC), *map(str, paths), "-o", str(out), *flags]
     else:
         cmd = [CXX, "-O2", "-std=c++17", *shared, "-I", str(CSRC), *map(str, paths), "-o",
                str(out), *flags]

@@ -16,10 +16,110 @@ from typing import Any
 import torch
 
 
+@dataclass(frozen=True)
+class LatentMixerSpec:
+    """A latent-attention mixer: queries and keys/values pass through low-rank latents; a head's
+    query/key has ``dim`` unrotated and ``rot_dim`` rotated channels (the rotated key part is one
+    vector shared by all heads), its value ``vdim`` channels.  Only the KV latent (``kv_rank``) and
+    the rotated key part are cached.  ``kv_from``: the layer whose cache entries this layer reads
+    instead of writing its own (it then has no KV down-projection)."""
+    heads: int
+    dim: int
+    rot_dim: int
+    vdim: int
+    kv_rank: int
+    q_rank: int
+    rope_base: float
+    rope_dims: int
+    scale: float
+    kv_from: int | None = None
+    sink: bool = True          # a learned per-head logit in the softmax denominator
+    out_gate: bool = True      # head outputs times sigmoid(W_g h)
+
+    @property
+    def entry(self) -> int:    # cached values per token
+        return self.kv_rank + self.rot_dim
+
+
+@dataclass(frozen=True)
+class FeedForwardSpec:
+    """``dense``: down(relu(up x)^2).  ``moe``: ``experts`` clamped gated units of width ``ff``, ``top``
+    per token out of the ``keep`` best of ``groups`` groups, sigmoid scores times ``route_scale``;
+    an always-on shared unit of width ``shared_ff`` (0 = none) with a per-token sigmoid gate."""
+    kind: str = "dense"
+    ff: int = 0
+    experts: int = 0
+    top: int = 0
+    groups: int = 1
+    keep: int = 1
+    route_scale: float = 1.0
+    limit: float = 0.0
+    shared_ff: int = 0
+    shared_limit: float = 0.0
+
+
+@dataclass(frozen=True)
+class LayerSpec:
+    type: str
+    mixer: LatentMixerSpec
+    mlp: FeedForwardSpec | None = None
+
+
+def zururax_layers(layers: list[dict]) -> tuple:
+    """The ``layers`` list of a Zururax config.json -> layer specs."""
+    out = []
+    for i, entry in enumerate(layers):
+        if entry["type"] != "latent_attention":
+            raise ValueError(f"layer {i}: unknown mixer type {entry['type']!r}")
+        m = entry["mixer"]
+        rot = m.get("rot") or {}
+        src = m.get("kv_from")
+        mixer = LatentMixerSpec(
+            heads=int(m["heads"]), dim=int(m["dim"]), rot_dim=int(m["rot_dim"]), vdim=int(m["vdim"]),
+            kv_rank=int(m["kv_rank"]), q_rank=int(m["q_rank"]), rope_base=float(rot.get("base", 10000.0)),
+            rope_dims=int(rot.get("dims", m["rot_dim"])), scale=float(m["scale"]),
+            kv_from=None if src is None else int(src))
+        if mixer.kv_from is not None:
+            if not 0 <= mixer.kv_from < i:
+                raise ValueError(f"layer {i}: kv_from must name an earlier layer")
+            s = out[mixer.kv_from].mixer
+            if s.kv_from is not None or (s.kv_rank, s.rot_dim) != (mixer.kv_rank, mixer.rot_dim):
+                raise ValueError(f"layer {i}: layer {mixer.kv_from} does not hold entries of this layer's shape")
+        f = entry.get("mlp")
+        mlp = None
+        if f is not None:
+            if f["kind"] == "dense":
+                mlp = FeedForwardSpec(kind="dense", ff=int(f["ff"]))
+            elif f["kind"] == "moe":
+                r, ex, sh = f["router"], f["expert"], f.get("shared")
+                g = r.get("groups") or {}
+                mlp = FeedForwardSpec(
+                    kind="moe", ff=int(ex["ff"]), experts=int(r["experts"]), top=int(r["top"]),
+                    groups=int(g.get("count", 1)), keep=int(g.get("keep", g.get("count", 1))),
+                    route_scale=float(r.get("scale", 1.0)), limit=float(ex["limit"]),
+                    shared_ff=int(sh["ff"]) if sh else 0, shared_limit=float(sh["limit"]) if sh else 0.0)
+            else:
+                raise ValueError(f"layer {i}: unknown feed-forward kind {f['kind']!r}")
+        out.append(LayerSpec("latent_attention", mixer, mlp))
+    return tuple(out)
+
+
+def zururax_config(name: str, vocab: int, width: int, layers: list[dict], embedding_scale: float = 1.0,
+                   norm_eps: float = 1e-5, max_position_embeddings: int = 8192) -> "ModelConfig":
+    specs = zururax_layers(layers)
+    return ModelConfig(
+        name=name, architecture="zururax", vocab_size=int(vocab), hidden_size=int(width),
+        intermediate_size=max([s.mlp.ff for s in specs if s.mlp] + [0]), num_layers=len(specs),
+        num_heads=max(s.mixer.heads for s in specs), num_kv_heads=1,
+        head_dim=max(s.mixer.dim + s.mixer.rot_dim for s in specs), norm_eps=float(norm_eps),
+        max_position_embeddings=max_position_embeddings, embedding_scale=float(embedding_scale),
+        layer_specs=specs)
+
+
 @dataclass
 class ModelConfig:
     name: str = "tiny-llama"
-    architecture: str = "llama"  # llama | mixtral | opt | gpt2
+    architecture: str = "llama"  # llama | mixtral | opt | gpt2 | zururax
     vocab_size: int = 512
     hidden_size: int = 256
     intermediate_size: int = 512
@@ -42,6 +142,9 @@ class ModelConfig:
     ffn_dim: int = 0
     pos_offset: int = 0
     activation: str = "relu"  # relu (OPT) | gelu_new (GPT-2)
+    # designs whose layers differ from one another list them (Zururax); empty = num_layers equal layers
+    layer_specs: tuple = ()
+    embedding_scale: float = 1.0
 
     @property
     def q_size(self) -> int:
@@ -54,12 +157,31 @@ class ModelConfig:
     def prefill_flops(self) -> tuple[float, float]:
         """(GEMM FLOPs per new token, attention FLOPs per (new token x context token) pair)."""
         h, i = self.hidden_size, self.intermediate_size
+        if self.layer_specs:
+            gemm = pair = 0.0
+            for s in self.layer_specs:
+                m, f = s.mixer, s.mlp
+                gemm += h * (m.q_rank + m.heads) + m.q_rank * m.heads * (m.dim + m.rot_dim) + m.heads * m.vdim * h
+                gemm += m.heads * m.kv_rank * (m.dim + m.vdim) + (h * m.entry if m.kv_from is None else 0)
+                pair += m.heads * (m.entry + m.kv_rank)
+                if f is not None:
+                    gemm += 2 * h * f.ff if f.kind == "dense" else 3 * h * (f.top * f.ff + f.shared_ff) + h * f.experts
+            return 2.0 * gemm, 2.0 * pair
         attn_w = h * (self.q_size + 2 * self.kv_size) + self.q_size * h
         mlp_w = 3 * h * i * max(1, self.num_experts_per_tok if self.num_experts else 1)
         return 2.0 * self.num_layers * (attn_w + mlp_w), 4.0 * self.num_layers * self.q_size
 
     def num_params(self) -> int:
         h, i, l_ = self.hidden_size, self.intermediate_size, self.num_layers
+        if self.layer_specs:
+            n = 2 * self.vocab_size * h
+            for s in self.layer_specs:
+                m, f = s.mixer, s.mlp
+                n += h * (m.q_rank + m.heads) + m.q_rank * m.heads * (m.dim + m.rot_dim) + m.heads * m.vdim * h
+                n += m.heads * m.kv_rank * (m.dim + m.vdim) + (h * m.entry if m.kv_from is None else 0)
+                if f is not None:
+                    n += 2 * h * f.ff if f.kind == "dense" else 3 * h * (f.experts * f.ff + f.shared_ff) + h * f.experts
+            return n
         attn = h * (self.q_size + 2 * self.kv_size) + self.q_size * h
         mlp = 3 * h * i * max(1, self.num_experts)
         emb = self.vocab_size * h * (1 if self.tie_word_embeddings else 2)
@@ -156,6 +278,41 @@ PRESETS: dict[str, ModelConfig] = {
                             max_position_embeddings=2048),
 }
 
+
+
+def _zx_mixer(heads, dim, rot_dim, vdim, kv_rank, q_rank, base=10000.0, kv_from=None):
+    m = {"heads": heads, "dim": dim, "rot_dim": rot_dim, "vdim": vdim, "kv_rank": kv_rank, "q_rank": q_rank,
+         "rot": {"base": base, "dims": rot_dim}, "scale": (dim + rot_dim) ** -0.5}
+    if kv_from is not None:
+        m["kv_from"] = kv_from
+    return m
+
+
+def _zx_moe(ff, experts, top, groups, keep, shared_ff, scale=1.0, limit=7.0):
+    return {"kind": "moe", "expert": {"ff": ff, "limit": limit},
+            "router": {"experts": experts, "top": top, "groups": {"count": groups, "keep": keep}, "scale": scale},
+            "shared": {"ff": shared_ff, "limit": limit} if shared_ff else None}
+
+
+def _zx_layer(mixer, mlp):
+    return {"type": "latent_attention", "mixer": mixer, "mlp": mlp}
+
+
+# Zururax at random weights: a small one for tests and smoke runs, and one with the layer shapes of a
+# mid-sized latent-attention mixture model (benchmarks; every second layer reads its neighbour's cache)
+PRESETS["tiny-zururax"] = zururax_config(
+    "tiny-zururax", 512, 192,
+    [_zx_layer(_zx_mixer(3, 16, 8, 24, 48, 40), {"kind": "dense", "ff": 320}),
+     _zx_layer(_zx_mixer(3, 16, 8, 24, 48, 40, kv_from=0), _zx_moe(48, 8, 2, 2, 1, 80, scale=1.5, limit=1.0)),
+     _zx_layer(_zx_mixer(2, 24, 16, 16, 64, 56, base=50000.0), _zx_moe(48, 6, 3, 3, 2, 0, scale=2.0, limit=2.0))],
+    embedding_scale=2.0, max_position_embeddings=4096)
+PRESETS["zururax-bench"] = zururax_config(
+    "zururax-bench", 32000, 4096,
+    [_zx_layer(_zx_mixer(32, 128, 64, 128, 512, 1536, kv_from=(i - 1 if i % 2 else None)),
+               {"kind": "dense", "ff": 14336} if i == 0 else _zx_moe(2048, 32, 4, 8, 4, 2048, scale=2.5))
+     for i in range(8)],
+    max_position_embeddings=32768)
+
 _ALIASES = {
     "meta-llama/meta-llama-3-8b": "llama-3-8b",
     "meta-llama/meta-llama-3-8b-instruct": "llama-3-8b",
@@ -181,6 +338,11 @@ _ALIASES = {
 
 
 def _from_hf_config(cfg: dict[str, Any], name: str) -> ModelConfig:
+    if str(cfg.get("architecture", "")).lower() == "zururax":
+        return zururax_config(name, cfg["vocab"], cfg["width"], cfg["layers"],
+                              embedding_scale=(cfg.get("embedding") or {}).get("scale", 1.0),
+                              norm_eps=(cfg.get("norm") or {}).get("eps", 1e-5),
+                              max_position_embeddings=int(cfg.get("max_positions", 32768)))
     arch = (cfg.get("architectures") or [""])[0].lower()
     mt = cfg.get("model_type", "").lower()
     if "opt" in (arch + mt):

@@ -228,6 +228,37 @@ class LLMEngine:
             pr["steps_" + kind] = n
         return outputs
 
+    def forced_step(self, entries: list[tuple[str, list[int], list[int]]],
+                    finished: list[str] | tuple = ()) -> torch.Tensor | None:
+        """One engine step whose batch the caller dictates: ``entries`` = (request id, its next tokens,
+        rows among them whose logits are wanted).  All entries run as one batch (single tokens of
+        requests that are under way as decode rows, everything else as prefill chunks) from what
+        earlier steps left in the cache; an unknown id starts a request.  ``finished`` requests give
+        their pages and slot back after the step.  Returns fp32 logits [wanted rows, vocab] in the
+        order of the entries and their wanted rows (None when nothing is wanted).  Nothing is
+        sampled and no prefix is reused: the step computes exactly the tokens it is given."""
+        from .scheduler import SchedulerOutput
+
+        out = SchedulerOutput()
+        seqs = []
+        for rid, tokens, want in entries:
+            req = self.requests.get(rid)
+            if req is None:
+                req = self.requests[rid] = Request(rid, [], SamplingParams(max_tokens=1))
+            s = self.scheduler.force(req, list(tokens), list(want))
+            (out.decodes if s.n == 1 and s.start > 0 else out.prefills).append(s)
+            seqs.append(s)
+        self.step_count += 1
+        res = self.runner.score(out)
+        for s in seqs:
+            self.scheduler.commit(s)
+        for rid in finished:
+            req = self.requests.pop(rid, None)
+            if req is not None:
+                self.scheduler.finish(req, "stop")
+        rows = [res[id(s)] for s in seqs if id(s) in res]
+        return torch.cat(rows, dim=0) if rows else None
+
     def _decode_run_length(self, out) -> int:
         """How many decode steps to launch back to back (``--num-scheduler-steps``): more than one
         only for a decode-only step of plain greedy rows with nothing waiting to be admitted, every

@@ -69,7 +69,12 @@ class ModelRunner:
         self.n_layers_local = len(self.model.layers)
         # channels per head as stored in the pool (heads of 64 are padded to the kernels' 128 on a GPU)
         self.kv_head_dim = ops.kv_head_dim(model_cfg.head_dim, device)
-        self.page_elems = self.n_layers_local * 2 * self.n_kv_local * PAGE * self.kv_head_dim
+        # one page of the pool: K and V of every local layer and KV head, unless the model lays its
+        # cache out itself (latent entries of the caching layers)
+        self.custom_pages = hasattr(self.model, "kv_page_shape")
+        self.page_dims = tuple(self.model.kv_page_shape()) if self.custom_pages else (
+            self.n_layers_local, 2, self.n_kv_local, PAGE * self.kv_head_dim)
+        self.page_elems = int(np.prod(self.page_dims))
         self.page_bytes = self.page_elems * torch.empty((), dtype=self.dtype).element_size()
         self.max_pages_per_seq = (self.max_model_len + PAGE - 1) // PAGE
         self.num_pages = self._plan_pages()
@@ -80,7 +85,7 @@ class ModelRunner:
         self.sampler = Sampler(device, cfg.seed)
         # graphs need the HIP attention kernels (the generic path reads lengths on the host)
         self.use_graphs = (device.type == "cuda" and not cfg.enforce_eager
-                           and self.kv_head_dim == ops.HEAD_DIM_HIP
+                           and getattr(self.model, "graph_capturable", self.kv_head_dim == ops.HEAD_DIM_HIP)
                            and (not self.distributed or self._tp_graphs_ready()))
         self._graphs: dict[int, dict] = {}
         self._prefill_graphs: dict[int, dict] = {}
@@ -148,6 +153,8 @@ class ModelRunner:
         of one of 8 MiB took the reload-bound benchmark phase from 450 to 432 output tok/s.  So
         the default of 0 picks 4 only for a large GPU pool on a replica without lower tiers and
         outside such transfers; with tiers it is the operator's call (few reloads: take it)."""
+        if self.custom_pages:
+            return 1
         g = int(self.cfg.kv_layer_groups)
         off, kvt = self.cfg.kv_offload, self.cfg.kv_transfer
         whole_pages = (off.enable_pd or kvt is not None) and not self.distributed
@@ -163,7 +170,7 @@ class ModelRunner:
         return max(1, g)
 
     def _alloc_pool(self):
-        shape = (self.num_pages, self.n_layers_local, 2, self.n_kv_local, PAGE * self.kv_head_dim)
+        shape = (self.num_pages, *self.page_dims)
         g = self._layer_groups()
         if g > 1:
             return ops.LayerGroupedPool([
@@ -207,7 +214,7 @@ class ModelRunner:
             log.info("KV pool: %d pages instead of %d so that peers can map it", pages, self.num_pages)
         self.num_pages = pages
         self._pool_dev_ptr, self.pool_ipc_handle = int(ptr), buf.raw.hex()
-        return raw.view(self.dtype).view(pages, self.n_layers_local, 2, self.n_kv_local, PAGE * self.kv_head_dim)
+        return raw.view(self.dtype).view(pages, *self.page_dims)
 
     def _free_exported_pool(self) -> None:
         """After every tensor view of the pool is gone."""
@@ -270,7 +277,9 @@ class ModelRunner:
             ids.append(r.prompt_ids[tok_idx] if tok_idx < r.prompt_len else r.output_ids[tok_idx - r.prompt_len])
             pos.append(tok_idx)
             slots.append(r.pages[tok_idx // PAGE] * PAGE + tok_idx % PAGE)
-            if s.samples:
+            if s.want is not None:
+                logits_rows.extend(row + w for w in s.want)
+            elif s.samples:
                 logits_rows.append(row)
                 sample_seqs.append(s)
             row += 1
@@ -286,7 +295,9 @@ class ModelRunner:
             pg = np.asarray(r.pages[first:(s.start + s.n - 1) // PAGE + 1], dtype=np.int64)
             slots.extend((pg[t // PAGE - first] * PAGE + t % PAGE).tolist())
             row += s.n
-            if s.samples:
+            if s.want is not None:
+                logits_rows.extend(row - s.n + w for w in s.want)
+            elif s.samples:
                 logits_rows.append(row - 1)
                 sample_seqs.append(s)
         plan = {"ids": ids, "pos": pos, "slots": slots, "logits_rows": logits_rows,
@@ -331,7 +342,9 @@ class ModelRunner:
                 cu.append(cu[-1] + q)
             meta.pre_cu_q = self._to_dev(cu, torch.int32)
             meta.pre_ctx_lens = self._to_dev(plan["pre_ctx"], torch.int32)
-            if self.device.type == "cuda":
+            if hasattr(self.model, "plan_prefill"):  # the model's attention kernels take a work list of their own
+                self.model.plan_prefill(meta, q_lens, plan["pre_ctx"], self._to_dev)
+            elif self.device.type == "cuda":
                 rows = ops.prefill_tile_rows(q_lens, self.model.n_q, self.model.n_kv)
                 ts, tq = ops.build_prefill_tiles(q_lens, self.model.n_q, self.model.n_kv, rows, plan["pre_ctx"])
                 cut = ops.plan_prefill_splits(ts, tq, q_lens, plan["pre_ctx"], self.model.n_q, self.model.n_kv, rows)
@@ -415,6 +428,32 @@ class ModelRunner:
         if self.distributed:
             check_collectives()  # the sampled tokens are on the host: every kernel of the step has run
         return list(zip(sample_seqs, toks, infos))
+
+    @torch.inference_mode()
+    def score(self, out: SchedulerOutput) -> dict[int, torch.Tensor]:
+        """Run one step without sampling: every sequence of ``out`` carries ``want``, the rows of its
+        chunk whose logits are asked for.  Returns ``{id(seq): fp32 logits [len(want), vocab]}``.  The
+        rows go through the same plan, batch assembly, model and kernels as a sampling step (eager
+        launches; single-rank replicas)."""
+        if out.empty:
+            return {}
+        if self.distributed:
+            raise RuntimeError("scoring steps run on single-rank replicas")
+        seqs = out.decodes + out.prefills
+        assert all(s.want is not None for s in seqs)
+        if self.device.type == "cuda":
+            ops.ensure_device()
+        self.step_kinds["eager"] += 1
+        plan, _ = self._plan(out.decodes, out.prefills)
+        _, logits = self._run_plan(plan)
+        res: dict[int, torch.Tensor] = {}
+        row = 0
+        for s in seqs:
+            k = len(s.want)
+            if k:
+                res[id(s)] = logits[row:row + k].float()
+            row += k
+        return res
 
     # ------------------------------------------------------------------ worker ranks
     def worker_loop(self) -> None:

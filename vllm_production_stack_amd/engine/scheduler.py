@@ -27,6 +27,8 @@ class ScheduledSeq:
     start: int  # tokens already in cache
     n: int  # rows this step
     samples: bool  # chunk reaches the end of the known tokens -> sample a new token
+    # scoring steps (``ModelRunner.score``): rows of this chunk whose logits are returned; nothing is sampled
+    want: list[int] | None = None
 
 
 @dataclass
@@ -259,6 +261,32 @@ class Scheduler:
             (out.decodes if n == 1 and req.num_computed > 0 else out.prefills).append(seq)
             budget -= n
         return out
+
+    # ------------------------------------------------------------------ dictated steps
+    def force(self, req: Request, tokens: list[int], want: list[int]) -> ScheduledSeq:
+        """A chunk the caller dictates instead of ``schedule()`` (replay of a recorded schedule,
+        scoring of given text): ``tokens`` continue ``req`` where its cache ends; a request seen for
+        the first time takes a sequence slot.  The rows get pages as scheduled rows do; with no page or
+        no slot left this raises, since nothing may be preempted behind the caller's back."""
+        if req not in self.running:
+            if len(self.running) >= self.max_num_seqs:
+                raise RuntimeError(f"all {self.max_num_seqs} sequence slots are taken")
+            if req in self.waiting:
+                self.waiting.remove(req)
+            req.state = RequestState.RUNNING
+            self.running.append(req)
+        if req.num_computed != req.num_tokens:
+            raise RuntimeError("a dictated chunk must start where the request's cache ends")
+        start, n = req.num_computed, len(tokens)
+        if n == 0 or start + n > self.max_model_len:
+            raise ValueError(f"chunk of {n} tokens at {start}: empty or past the context limit {self.max_model_len}")
+        if any(not 0 <= w < n for w in want):
+            raise ValueError("wanted rows lie outside the chunk")
+        req.prompt_ids.extend(tokens)
+        if not self._ensure_pages(req, start + n):
+            del req.prompt_ids[start:]
+            raise MemoryError(f"KV pool exhausted: {self.bm.num_free()} pages free")
+        return ScheduledSeq(req, start, n, False, list(want))
 
     def _unadmit(self, req: Request) -> None:
         if req.load_event is None:

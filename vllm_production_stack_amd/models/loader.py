@@ -17,6 +17,7 @@ from ..engine.config import ModelConfig
 from ..parallel.state import get_tp
 from .opt import OPTModel
 from .transformer import LayerWeights, TransformerModel
+from .zururax import ZururaxModel
 
 
 def build_model(cfg: ModelConfig, dtype: torch.dtype, device: torch.device, max_model_len: int,
@@ -24,6 +25,8 @@ def build_model(cfg: ModelConfig, dtype: torch.dtype, device: torch.device, max_
                 expert_parallel: bool = False):
     if cfg.architecture in ("opt", "gpt2"):
         model = OPTModel(cfg, dtype, device, max_model_len)
+    elif cfg.architecture == "zururax":
+        model = ZururaxModel(cfg, dtype, device, max_model_len)
     else:
         model = TransformerModel(cfg, dtype, device, max_model_len, expert_parallel=expert_parallel)
     has_weights = ckpt_dir is not None and any(Path(ckpt_dir).glob("*.safetensors"))
@@ -53,6 +56,8 @@ def _iter_safetensors(ckpt_dir: Path):
 def load_hf_weights(model, ckpt_dir: Path) -> None:
     if isinstance(model, OPTModel):
         (_load_gpt2 if model.cfg.architecture == "gpt2" else _load_opt)(model, ckpt_dir)
+    elif isinstance(model, ZururaxModel):
+        _load_zururax(model, ckpt_dir)
     else:
         _load_llama(model, ckpt_dir)
 
@@ -216,3 +221,110 @@ def _load_gpt2(model: OPTModel, ckpt_dir: Path) -> None:
             if m and m.group(2) in table:
                 key, transpose = table[m.group(2)]
                 model.layers[int(m.group(1))][key].copy_(t.t() if transpose else t)
+
+
+def _load_zururax(model: ZururaxModel, ckpt_dir: Path) -> None:
+    """Zururax checkpoints: ``embed``, ``l<i>.norm1|norm2``, ``l<i>.mix.{dq, dq.norm, uq, dkv, dkv.norm, uk, uv,
+    sink, g, o}``, ``l<i>.mlp.{up, down}`` or ``l<i>.mlp.{router, e<k>.{gate, up, down}, shared.{gate, up, down,
+    sg}}``, ``final.norm``, ``head``; linear weights are [out, in].  Every tensor the model holds must
+    be found, and every tensor of the file must have a place."""
+    pat = re.compile(r"l(\d+)\.(.+)")
+    expert = re.compile(r"mlp\.e(\d+)\.(gate|up|down)")
+    seen: set[str] = set()
+
+    def put(dst: torch.Tensor, src: torch.Tensor, what: str) -> None:
+        if tuple(dst.shape) != tuple(src.shape):
+            raise ValueError(f"{what}: checkpoint shape {tuple(src.shape)}, model expects {tuple(dst.shape)}")
+        dst.copy_(src.to(dst.dtype))
+
+    for name, t in _iter_safetensors(ckpt_dir):
+        seen.add(name)
+        if name == "embed":
+            put(model.embed, t, name)
+        elif name == "head":
+            put(model.lm_head, t, name)
+        elif name == "final.norm":
+            put(model.norm, t, name)
+        else:
+            mt = pat.match(name)
+            if not mt or int(mt.group(1)) >= len(model.layers):
+                raise ValueError(f"unexpected tensor {name!r}")
+            lw = model.layers[int(mt.group(1))]
+            sub = mt.group(2)
+            m, f = lw.spec.mixer, lw.spec.mlp
+            own = m.kv_from is None
+            me = expert.fullmatch(sub)
+            if sub == "norm1":
+                put(lw.norm1, t, name)
+            elif sub == "norm2" and f is not None:
+                put(lw.norm2, t, name)
+            elif sub == "mix.dq":
+                put(lw.w_in[:m.q_rank], t, name)
+            elif sub == "mix.dkv" and own:
+                put(lw.w_in[m.q_rank:m.q_rank + m.entry], t, name)
+            elif sub == "mix.g" and m.out_gate:
+                put(lw.w_in[lw.w_in.shape[0] - m.heads:], t, name)
+            elif sub == "mix.dq.norm":
+                put(lw.dq_norm, t, name)
+            elif sub == "mix.dkv.norm" and own:
+                put(lw.dkv_norm, t, name)
+            elif sub == "mix.uq":
+                put(lw.w_uq, t, name)
+            elif sub == "mix.uk":
+                put(lw.w_uk.view(m.heads * m.dim, m.kv_rank), t, name)
+            elif sub == "mix.uv":
+                put(lw.w_uv.view(m.heads * m.vdim, m.kv_rank), t, name)
+            elif sub == "mix.sink" and m.sink:
+                put(lw.sink, t, name)
+            elif sub == "mix.o":
+                put(lw.w_o, t, name)
+            elif sub == "mlp.up" and f is not None and f.kind == "dense":
+                put(lw.w_up, t, name)
+            elif sub == "mlp.down" and f is not None and f.kind == "dense":
+                put(lw.w_down, t, name)
+            elif sub == "mlp.router" and f is not None and f.kind == "moe":
+                put(lw.router[:f.experts], t, name)
+            elif me and f is not None and f.kind == "moe" and int(me.group(1)) < f.experts:
+                e, which = int(me.group(1)), me.group(2)
+                if which == "gate":
+                    put(lw.w13[e, :f.ff], t, name)
+                elif which == "up":
+                    put(lw.w13[e, f.ff:], t, name)
+                else:
+                    put(lw.w2[e], t, name)
+            elif sub.startswith("mlp.shared.") and f is not None and f.shared_ff:
+                which = sub[len("mlp.shared."):]
+                if which == "gate":
+                    put(lw.w_sh13[:f.shared_ff], t, name)
+                elif which == "up":
+                    put(lw.w_sh13[f.shared_ff:], t, name)
+                elif which == "down":
+                    put(lw.w_sh2, t, name)
+                elif which == "sg":
+                    put(lw.router[f.experts:], t, name)
+                else:
+                    raise ValueError(f"unexpected tensor {name!r}")
+            else:
+                raise ValueError(f"unexpected tensor {name!r}")
+    want = {"embed", "head", "final.norm"}
+    for i, lw in enumerate(model.layers):
+        m, f = lw.spec.mixer, lw.spec.mlp
+        want |= {f"l{i}.norm1", f"l{i}.mix.dq", f"l{i}.mix.dq.norm", f"l{i}.mix.uq", f"l{i}.mix.uk", f"l{i}.mix.uv",
+                 f"l{i}.mix.o"}
+        if m.kv_from is None:
+            want |= {f"l{i}.mix.dkv", f"l{i}.mix.dkv.norm"}
+        if m.sink:
+            want.add(f"l{i}.mix.sink")
+        if m.out_gate:
+            want.add(f"l{i}.mix.g")
+        if f is not None:
+            want.add(f"l{i}.norm2")
+            if f.kind == "dense":
+                want |= {f"l{i}.mlp.up", f"l{i}.mlp.down"}
+            else:
+                want.add(f"l{i}.mlp.router")
+                want |= {f"l{i}.mlp.e{e}.{k}" for e in range(f.experts) for k in ("gate", "up", "down")}
+                if f.shared_ff:
+                    want |= {f"l{i}.mlp.shared.{k}" for k in ("gate", "up", "down", "sg")}
+    if want - seen:
+        raise ValueError(f"checkpoint lacks {sorted(want - seen)[:8]}")

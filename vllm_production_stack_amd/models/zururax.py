@@ -1,0 +1,236 @@
+"""Zururax: a decoder whose layers are listed one by one in the configuration.
+
+Every layer is pre-norm around a latent-attention mixer and an optional feed-forward (dense
+squared-ReLU, or a mixture of clamped gated units with group-limited sigmoid routing and a gated
+shared unit).  The residual stream is fp32 whatever the activation dtype; a projection's output is
+added to it by the norm kernel that follows (``ops.add_rms_norm``), as the framework's other
+decoders do with their bf16 stream.
+
+Latent attention over the paged pool: a token's cache entry is its RMS-normed KV latent and the
+rotated key part shared by all heads (``kv_rank + rot_dim`` values; layers with ``kv_from`` read the
+entries of the layer they name and own no cache).  Keys and values are never expanded: a head's
+unrotated query is carried into latent space (q W_uk, one batched matrix product), the attention
+kernel scores it against the entries and returns the probability-weighted latent, and W_uv takes
+that to the head's value space.  All heads then share one key/value stream per token.
+
+The input projections of a mixer (query latent | KV latent and shared key part | output-gate logits)
+are one fused matrix, as are gate | up of every gated unit; the router's matrix (with the shared
+unit's gate row appended) is fp32 and its product is a true fp32 one.
+"""
+
+from __future__ import annotations
+
+import torch
+import torch.nn.functional as F
+
+from .. import ops
+from ..engine.config import FeedForwardSpec, LatentMixerSpec, ModelConfig
+from ..ops.reference import PAGE
+from ..parallel.state import get_pp, get_tp
+from .batch import BatchMeta
+
+GLU_ALPHA = 1.702   # the gated units' sigmoid slope
+GLU_UP_BIAS = 1.0   # and the offset of their linear branch
+
+
+class ZururaxLayer:
+    __slots__ = ("spec", "norm1", "norm2", "w_in", "dq_norm", "dkv_norm", "w_uq", "w_uk", "w_uv", "sink", "w_o",
+                 "w_up", "w_down", "router", "w13", "w2", "w_sh13", "w_sh2", "cache_offset", "cos_sin")
+
+    def __init__(self, spec):
+        for s in self.__slots__:
+            setattr(self, s, None)
+        self.spec = spec
+
+
+class ZururaxModel:
+    graph_capturable = False  # the expert loop reads the per-expert row counts on the host
+
+    def __init__(self, cfg: ModelConfig, dtype: torch.dtype, device: torch.device, max_model_len: int):
+        if get_tp().size != 1 or get_pp().size != 1:
+            raise ValueError("Zururax runs on single-GPU replicas (no tensor / pipeline parallel layout yet)")
+        if dtype not in (torch.bfloat16, torch.float32):
+            raise ValueError("Zururax runs in bfloat16 or float32")
+        self.cfg = cfg
+        self.dtype = dtype
+        self.device = device
+        self.max_model_len = max_model_len
+        self.specs = cfg.layer_specs
+        self.n_q = cfg.num_heads
+        self.n_kv = 1
+        self.head_dim = cfg.head_dim
+        self.tp_size = 1
+        self.lora = None
+        self.layers: list[ZururaxLayer] = []
+        self.embed = self.norm = self.lm_head = None
+        self.layer_probe = None  # callable(layer index, fp32 residual stream after the layer) for tests
+        # where each caching layer's entries start inside a page, in elements
+        off = 0
+        self.cache_offsets: dict[int, int] = {}
+        for i, s in enumerate(self.specs):
+            if s.mixer.kv_from is None:
+                self.cache_offsets[i] = off
+                off += PAGE * s.mixer.entry
+        self.page_elems = off
+        self._tables: dict[tuple, torch.Tensor] = {}
+
+    # ------------------------------------------------------------------ cache layout
+    def kv_page_shape(self) -> tuple:
+        """Shape of one page of the KV pool (the runner allocates [pages, *shape])."""
+        return (self.page_elems,)
+
+    def _cos_sin(self, m: LatentMixerSpec) -> torch.Tensor:
+        key = (m.rope_base, m.rope_dims)
+        t = self._tables.get(key)
+        if t is None:
+            t = self._tables[key] = ops.build_cos_sin(m.rope_dims, self.max_model_len, m.rope_base, None,
+                                                      device=self.device)
+        return t
+
+    # ------------------------------------------------------------------ weights
+    def _alloc(self, gen, *shape, std=None, dtype=None, ones=False):
+        dtype = dtype or self.dtype
+        if ones:
+            return torch.ones(shape, dtype=dtype, device=self.device)
+        t = torch.empty(shape, dtype=torch.float32, device=self.device)
+        t.normal_(0.0, std if std is not None else shape[-1] ** -0.5, generator=gen)
+        return t.to(dtype)
+
+    def init_random(self, seed: int = 0) -> None:
+        """Allocates every tensor in the layout the forward pass uses; a checkpoint overwrites them.
+        Projections are drawn with std 1/sqrt(fan-in) so that activations stay of order one."""
+        cfg = self.cfg
+        w = cfg.hidden_size
+        g = torch.Generator(device=self.device).manual_seed(seed)
+        f32 = torch.float32
+        self.embed = self._alloc(g, cfg.vocab_size, w, std=1.0)
+        self.layers = []
+        for i, s in enumerate(self.specs):
+            m, f = s.mixer, s.mlp
+            lw = ZururaxLayer(s)
+            own = m.kv_from is None
+            lw.norm1 = self._alloc(g, w, ones=True, dtype=f32)
+            lw.w_in = self._alloc(g, m.q_rank + (m.entry if own else 0) + (m.heads if m.out_gate else 0), w)
+            lw.dq_norm = self._alloc(g, m.q_rank, ones=True, dtype=f32)
+            lw.dkv_norm = self._alloc(g, m.kv_rank, ones=True, dtype=f32) if own else None
+            lw.w_uq = self._alloc(g, m.heads * (m.dim + m.rot_dim), m.q_rank)
+            lw.w_uk = self._alloc(g, m.heads, m.dim, m.kv_rank)
+            lw.w_uv = self._alloc(g, m.heads, m.vdim, m.kv_rank)
+            lw.sink = self._alloc(g, m.heads, std=1.0, dtype=f32) if m.sink else None
+            lw.w_o = self._alloc(g, w, m.heads * m.vdim)
+            lw.cache_offset = self.cache_offsets[i if own else m.kv_from]
+            lw.cos_sin = self._cos_sin(m)
+            if f is not None:
+                lw.norm2 = self._alloc(g, w, ones=True, dtype=f32)
+                if f.kind == "dense":
+                    lw.w_up = self._alloc(g, f.ff, w)
+                    lw.w_down = self._alloc(g, w, f.ff)
+                else:
+                    lw.router = self._alloc(g, f.experts + (1 if f.shared_ff else 0), w, dtype=f32)
+                    lw.w13 = self._alloc(g, f.experts, 2 * f.ff, w)
+                    lw.w2 = self._alloc(g, f.experts, w, f.ff)
+                    if f.shared_ff:
+                        lw.w_sh13 = self._alloc(g, 2 * f.shared_ff, w)
+                        lw.w_sh2 = self._alloc(g, w, f.shared_ff)
+            self.layers.append(lw)
+        self.norm = self._alloc(g, w, ones=True, dtype=f32)
+        self.lm_head = self._alloc(g, cfg.vocab_size, w)
+
+    def weight_tensors(self):
+        for t in (self.embed, self.norm, self.lm_head):
+            if t is not None:
+                yield t
+        for lw in self.layers:
+            for s in ZururaxLayer.__slots__:
+                t = getattr(lw, s)
+                if isinstance(t, torch.Tensor) and s != "cos_sin":
+                    yield t
+
+    def weight_bytes(self) -> int:
+        return sum(t.numel() * t.element_size() for t in self.weight_tensors())
+
+    # ------------------------------------------------------------------ batch description
+    def plan_prefill(self, meta: BatchMeta, q_lens: list[int], ctx_lens: list[int], to_dev) -> None:
+        """Which sequence of the prefill part each prefill row belongs to."""
+        seq: list[int] = []
+        for i, n in enumerate(q_lens):
+            seq.extend([i] * n)
+        meta.pre_row_seq = to_dev(seq, torch.int32)
+
+    # ------------------------------------------------------------------ forward
+    def _mixer(self, lw: ZururaxLayer, h: torch.Tensor, pool, meta: BatchMeta) -> torch.Tensor:
+        m: LatentMixerSpec = lw.spec.mixer
+        eps = self.cfg.norm_eps
+        t = h.shape[0]
+        proj = F.linear(h, lw.w_in)
+        col = m.q_rank
+        cq = ops.rms_norm_rows(proj[:, :col], lw.dq_norm, eps)
+        q = F.linear(cq, lw.w_uq).view(t, m.heads, m.dim + m.rot_dim)
+        ops.rope_pairs(q, meta.positions, lw.cos_sin, m.dim, m.rope_dims)
+        if m.kv_from is None:
+            ops.latent_kv_write(proj[:, col:col + m.entry], lw.dkv_norm, meta.positions, meta.slots, lw.cos_sin, pool,
+                                lw.cache_offset, m.kv_rank, m.rot_dim, m.rope_dims, eps)
+            col += m.entry
+        # [heads, T, dim] x [heads, dim, kv_rank]: the unrotated query in latent space
+        q_lat = torch.bmm(q[:, :, :m.dim].transpose(0, 1), lw.w_uk).transpose(0, 1)
+        q_rot = q[:, :, m.dim:]
+        o_lat = torch.empty((t, m.heads, m.kv_rank), dtype=h.dtype, device=h.device)
+        nd = meta.num_decode
+        if nd > 0:
+            ops.latent_attention(q_lat[:nd], q_rot[:nd], pool, lw.cache_offset, meta.dec_block_tables, None,
+                                 meta.positions[:nd], lw.sink, m.scale, out=o_lat[:nd])
+        if meta.num_prefill_seqs > 0:
+            ops.latent_attention(q_lat[nd:], q_rot[nd:], pool, lw.cache_offset, meta.pre_block_tables,
+                                 meta.pre_row_seq, meta.positions[nd:], lw.sink, m.scale, out=o_lat[nd:])
+        # [heads, T, kv_rank] x [heads, kv_rank, vdim] -> [T, heads, vdim]
+        o = torch.bmm(o_lat.transpose(0, 1), lw.w_uv.transpose(1, 2)).transpose(0, 1).contiguous()
+        if m.out_gate:
+            ops.sigmoid_gate(o, proj[:, col:col + m.heads])
+        return F.linear(o.view(t, m.heads * m.vdim), lw.w_o)
+
+    def _moe(self, lw: ZururaxLayer, h: torch.Tensor, residual: torch.Tensor) -> None:
+        """Adds the mixture's output for rows h into the fp32 residual stream."""
+        f: FeedForwardSpec = lw.spec.mlp
+        t = h.shape[0]
+        logits = F.linear(h.float(), lw.router)  # a true fp32 product
+        w, ids, gate = ops.group_topk(logits, f.experts, f.groups, f.keep, f.top, f.route_scale, extra=f.shared_ff > 0)
+        shared = None
+        if f.shared_ff:
+            shared = F.linear(ops.glu_clamp(F.linear(h, lw.w_sh13), f.shared_limit, GLU_ALPHA, GLU_UP_BIAS), lw.w_sh2)
+        offsets, pos, sorted_tok = ops.moe_align(ids, f.experts)
+        xs = ops.gather_rows(h, sorted_tok)
+        ys = torch.empty((t * f.top, h.shape[1]), dtype=h.dtype, device=h.device)
+        off = offsets.tolist()
+        for e in range(f.experts):
+            a, b = off[e], off[e + 1]
+            if b > a:
+                act = ops.glu_clamp(F.linear(xs[a:b], lw.w13[e]), f.limit, GLU_ALPHA, GLU_UP_BIAS)
+                torch.matmul(act, lw.w2[e].t(), out=ys[a:b])
+        ops.moe_finish(residual, ys, w, pos, shared, gate)
+
+    def forward(self, input_ids: torch.Tensor, pool: torch.Tensor, meta: BatchMeta) -> torch.Tensor:
+        """Final-normed hidden states of ``meta.logits_rows`` ([num_out, width], activation dtype)."""
+        cfg = self.cfg
+        eps = cfg.norm_eps
+        x = ops.embed_scale(input_ids, self.embed, cfg.embedding_scale)  # fp32 residual stream
+        d = None  # a projection output not yet added to the stream
+        for i, lw in enumerate(self.layers):
+            h = ops.add_rms_norm(x, d, lw.norm1, eps, self.dtype)
+            d = self._mixer(lw, h, pool, meta)
+            f = lw.spec.mlp
+            if f is not None:
+                h = ops.add_rms_norm(x, d, lw.norm2, eps, self.dtype)
+                d = None
+                if f.kind == "dense":
+                    d = F.linear(ops.relu_sq(F.linear(h, lw.w_up)), lw.w_down)
+                else:
+                    self._moe(lw, h, x)
+            if self.layer_probe is not None:
+                self.layer_probe(i, x if d is None else x + d.float())
+        if meta.logits_rows is not None:
+            x = x.index_select(0, meta.logits_rows)
+            d = None if d is None else d.index_select(0, meta.logits_rows)
+        return ops.add_rms_norm(x, d, self.norm, eps, self.dtype)
+
+    def compute_logits(self, hidden: torch.Tensor) -> torch.Tensor:
+        return F.linear(hidden, self.lm_head)

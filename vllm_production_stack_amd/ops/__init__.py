@@ -37,6 +37,9 @@ def _kernels():
             "vpsa_rans_decode", "vpsa_sample", "vpsa_grouped_gemm", "vpsa_packed_gemm",
             "vpsa_packed_gemm_splits", "vpsa_set_packed_target", "vpsa_dense_decode_attention", "vpsa_dense_attention",
             "vpsa_tile_gemm", "vpsa_tile_gemm_debug", "vpsa_paged_prefill_split",
+            "vpsa_embed_scale", "vpsa_add_rmsnorm", "vpsa_rmsnorm_rows", "vpsa_latent_kv_write", "vpsa_rope_pairs",
+            "vpsa_latent_attention", "vpsa_sigmoid_gate", "vpsa_relu_sq", "vpsa_glu_clamp", "vpsa_group_topk",
+            "vpsa_gather_rows", "vpsa_moe_finish",
         ):
             getattr(lib, name).restype = c_int
         lib.vpsa_prefill_split_record_bytes.restype = c_long
@@ -1310,3 +1313,8 @@ def lora_expand(h, bs, slots, y, r_pad):
                                      c_int(r_pad), c_int(bs[0].shape[0]), _stream())
     _check(rc, "lora_expand")
     return y
+
+
+# --------------------------------------------------------------------------- latent attention, group routing, fp32 residual
+from .latent import (add_rms_norm, embed_scale, gather_rows, glu_clamp, group_topk, latent_attention,  # noqa: E402,F401
+                     latent_kv_write, moe_finish, relu_sq, rms_norm_rows, rope_pairs, sigmoid_gate)

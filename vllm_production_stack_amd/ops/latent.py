@@ -1,0 +1,238 @@
+"""Ops of decoders with a 32-bit residual stream, latent attention and group-limited sigmoid
+routing (``csrc/kernels/latent.hip``).  Device tensors run the HIP kernels in bf16 or fp32
+activations; CPU tensors run the PyTorch definitions of ``reference.py``.
+
+The latent KV pool is ``[pages, page_elems]``: a page holds, for every caching layer, PAGE entries
+of ``rank + rot`` values (RMS-normed latent | rotated shared key part) starting ``offset`` elements
+into the page, so a page's whole depth stays one contiguous run.
+"""
+
+from __future__ import annotations
+
+from ctypes import c_float, c_int, c_long, c_void_p
+
+import torch
+
+from . import reference
+from .reference import PAGE
+
+_DT = {torch.bfloat16: 0, torch.float32: 1}
+
+
+def _ops():
+    from .. import ops
+
+    return ops
+
+
+def _dt(*ts) -> int:
+    d = None
+    for t in ts:
+        if t is None:
+            continue
+        if not t.is_cuda or t.dtype not in _DT:
+            raise TypeError("latent kernels take bf16 or fp32 device tensors")
+        if d is not None and _DT[t.dtype] != d:
+            raise TypeError("latent kernels: mixed activation dtypes")
+        d = _DT[t.dtype]
+    return d
+
+
+def _f32(*ts):
+    for t in ts:
+        if t is not None and (t.dtype != torch.float32 or not t.is_contiguous()):
+            raise TypeError("expected a contiguous fp32 tensor")
+
+
+def _rows(t) -> bool:  # a 2-D view whose rows are contiguous runs
+    return t.dim() == 2 and t.stride(1) == 1
+
+
+def embed_scale(ids, embed, scale: float):
+    """fp32 [T, width] = embed[ids] * scale."""
+    if not embed.is_cuda:
+        return reference.embed_scale(ids, embed, scale)
+    o = _ops()
+    assert ids.dtype == torch.int64 and embed.is_contiguous()
+    out = torch.empty((ids.shape[0], embed.shape[1]), dtype=torch.float32, device=embed.device)
+    o._check(o._kernels().vpsa_embed_scale(o._p(ids), o._p(embed), o._p(out), c_int(ids.shape[0]),
+                                           c_int(embed.shape[1]), c_float(scale), c_int(_dt(embed)), o._stream()),
+             "embed_scale")
+    return out
+
+
+def add_rms_norm(residual, delta, weight, eps: float, out_dtype, want_out: bool = True):
+    """residual (fp32, in place) += delta; returns rmsnorm(residual) * weight in ``out_dtype``."""
+    if not residual.is_cuda:
+        return reference.add_rms_norm(residual, delta, weight, eps, out_dtype, want_out)
+    o = _ops()
+    _f32(residual, weight)
+    t, n = residual.shape
+    assert delta is None or (_rows(delta) and delta.shape == residual.shape and delta.dtype == out_dtype)
+    y = torch.empty((t, n), dtype=out_dtype, device=residual.device) if want_out else None
+    if y is None and delta is None:
+        return None
+    o._check(o._kernels().vpsa_add_rmsnorm(o._p(residual), o._p(delta), c_long(delta.stride(0) if delta is not None else 0),
+                                           o._p(weight), o._p(y), c_long(n), c_int(t), c_int(n), c_float(eps),
+                                           c_int(_DT[out_dtype]), o._stream()), "add_rms_norm")
+    return y
+
+
+def rms_norm_rows(x, weight, eps: float):
+    """rmsnorm over the columns of a 2-D view (a column range of a wider projection output)."""
+    if not x.is_cuda:
+        return reference.rms_norm_rows(x, weight, eps)
+    o = _ops()
+    _f32(weight)
+    assert _rows(x) and weight.numel() == x.shape[1]
+    y = torch.empty(x.shape, dtype=x.dtype, device=x.device)
+    o._check(o._kernels().vpsa_rmsnorm_rows(o._p(x), c_long(x.stride(0)), o._p(weight), o._p(y), c_long(x.shape[1]),
+                                            c_int(x.shape[0]), c_int(x.shape[1]), c_float(eps), c_int(_dt(x)),
+                                            o._stream()), "rms_norm_rows")
+    return y
+
+
+def _layer_base(pool, offset: int, entry: int):
+    assert pool.dim() == 2 and pool.stride(1) == 1 and offset + PAGE * entry <= pool.shape[1]
+    return c_void_p(pool.data_ptr() + offset * pool.element_size())
+
+
+def latent_kv_write(x, weight, positions, slots, cos_sin, pool, offset: int, rank: int, rot: int, rot_dims: int,
+                    eps: float):
+    """Rows of x [T, rank + rot] (a view) -> cache entries: RMS-normed latent | rotated key part."""
+    if not x.is_cuda:
+        return reference.latent_kv_write(x, weight, positions, slots, cos_sin, pool, offset, rank, rot, rot_dims, eps)
+    o = _ops()
+    _f32(weight, cos_sin)
+    assert _rows(x) and x.shape[1] == rank + rot and positions.dtype == torch.int32 and slots.dtype == torch.int64
+    assert cos_sin.shape[1] == rot_dims and weight.numel() == rank
+    o._check(o._kernels().vpsa_latent_kv_write(o._p(x), c_long(x.stride(0)), o._p(weight), o._p(positions), o._p(slots),
+                                               o._p(cos_sin), _layer_base(pool, offset, rank + rot),
+                                               c_long(pool.stride(0)), c_int(x.shape[0]), c_int(rank), c_int(rot),
+                                               c_int(rot_dims), c_float(eps), c_int(_dt(x, pool)), o._stream()),
+             "latent_kv_write")
+
+
+def rope_pairs(q, positions, cos_sin, col0: int, rot_dims: int):
+    """Interleaved-pair rotary embedding of columns [col0, col0 + rot_dims) of every head of
+    q [T, heads, d], in place.  cos_sin [max_pos, rot_dims] = cos | sin of the rot_dims / 2 angles."""
+    if not q.is_cuda:
+        return reference.rope_pairs(q, positions, cos_sin, col0, rot_dims)
+    o = _ops()
+    _f32(cos_sin)
+    assert q.dim() == 3 and q.stride(2) == 1 and positions.dtype == torch.int32 and cos_sin.shape[1] == rot_dims
+    assert col0 + rot_dims <= q.shape[2]
+    o._check(o._kernels().vpsa_rope_pairs(o._p(q), c_long(q.stride(0)), c_long(q.stride(1)), o._p(positions),
+                                          o._p(cos_sin), c_int(q.shape[0]), c_int(q.shape[1]), c_int(col0),
+                                          c_int(rot_dims), c_int(_dt(q)), o._stream()), "rope_pairs")
+
+
+def latent_attention(q_lat, q_rot, pool, offset: int, block_tables, row_seq, positions, sink, scale: float, out=None):
+    """Causal attention of query rows over their sequences' cache entries, in latent space.
+
+    q_lat [T, heads, rank] and q_rot [T, heads, rot] (views with contiguous last dim); row ``i``
+    belongs to sequence ``row_seq[i]`` (``None``: row i is sequence i) whose pages are
+    ``block_tables[seq]`` and sees entries 0 .. positions[i].  ``sink`` [heads] fp32 or None: a logit
+    that joins the softmax denominator only.  Returns [T, heads, rank]."""
+    t, heads, rank = q_lat.shape
+    if out is None:
+        out = torch.empty((t, heads, rank), dtype=q_lat.dtype, device=q_lat.device)
+    if t == 0:
+        return out
+    if not q_lat.is_cuda:
+        return reference.latent_attention(q_lat, q_rot, pool, offset, block_tables, row_seq, positions, sink, scale, out)
+    o = _ops()
+    rot = q_rot.shape[2]
+    _f32(sink)
+    assert q_lat.stride(2) == 1 and q_rot.stride(2) == 1 and out.stride(2) == 1 and q_rot.shape[:2] == (t, heads)
+    assert block_tables.dtype == torch.int32 and block_tables.stride(1) == 1 and positions.dtype == torch.int32
+    assert row_seq is None or (row_seq.dtype == torch.int32 and row_seq.numel() == t)
+    o._check(o._kernels().vpsa_latent_attention(
+        o._p(q_lat), c_long(q_lat.stride(0)), c_long(q_lat.stride(1)), o._p(q_rot), c_long(q_rot.stride(0)),
+        c_long(q_rot.stride(1)), _layer_base(pool, offset, rank + rot), c_long(pool.stride(0)), o._p(block_tables),
+        c_int(block_tables.stride(0)), o._p(row_seq), o._p(positions), o._p(sink), o._p(out), c_long(out.stride(0)),
+        c_long(out.stride(1)), c_int(t), c_int(heads), c_int(rank), c_int(rot), c_float(scale),
+        c_int(_dt(q_lat, q_rot, pool, out)), o._stream()), "latent_attention")
+    return out
+
+
+def sigmoid_gate(y, g):
+    """y [T, heads, v] (contiguous, in place) *= sigmoid(g [T, heads]) (a view of a wider projection)."""
+    if not y.is_cuda:
+        return reference.sigmoid_gate(y, g)
+    o = _ops()
+    assert y.is_contiguous() and g.stride(1) == 1 and g.shape == y.shape[:2]
+    o._check(o._kernels().vpsa_sigmoid_gate(o._p(y), o._p(g), c_long(g.stride(0)), c_int(y.shape[0]), c_int(y.shape[1]),
+                                            c_int(y.shape[2]), c_int(_dt(y, g)), o._stream()), "sigmoid_gate")
+    return y
+
+
+def relu_sq(x):
+    if not x.is_cuda:
+        return reference.relu_sq(x)
+    o = _ops()
+    assert x.is_contiguous()
+    y = torch.empty_like(x)
+    o._check(o._kernels().vpsa_relu_sq(o._p(x), o._p(y), c_long(x.numel()), c_int(_dt(x)), o._stream()), "relu_sq")
+    return y
+
+
+def glu_clamp(x, limit: float, alpha: float = 1.702, up_bias: float = 1.0):
+    """x [rows, 2 I] = gate | up  ->  min(g, limit) * sigmoid(alpha min(g, limit)) * (clamp(u, +-limit) + up_bias)."""
+    if not x.is_cuda:
+        return reference.glu_clamp(x, limit, alpha, up_bias)
+    o = _ops()
+    assert _rows(x) and x.shape[1] % 2 == 0
+    inter = x.shape[1] // 2
+    y = torch.empty((x.shape[0], inter), dtype=x.dtype, device=x.device)
+    o._check(o._kernels().vpsa_glu_clamp(o._p(x), c_long(x.stride(0)), o._p(y), c_int(x.shape[0]), c_int(inter),
+                                         c_float(limit), c_float(alpha), c_float(up_bias), c_int(_dt(x)), o._stream()),
+             "glu_clamp")
+    return y
+
+
+def group_topk(logits, experts: int, groups: int, keep: int, topk: int, route_scale: float, extra: bool = False):
+    """Router logits fp32 [T, >= experts (+1)] -> (weights fp32 [T, topk], ids int32 [T, topk], extra).
+
+    Scores are sigmoids; experts form ``groups`` equal runs of neighbours, a group scores the sum of
+    its two largest scores, and only experts of the ``keep`` best groups can be chosen; weights are
+    the chosen scores times ``route_scale``.  ``extra``: column ``experts`` is one more logit per
+    token, returned as its sigmoid (a shared unit's gate)."""
+    if not logits.is_cuda:
+        return reference.group_topk(logits, experts, groups, keep, topk, route_scale, extra)
+    o = _ops()
+    _f32(logits)
+    t = logits.shape[0]
+    w = torch.empty((t, topk), dtype=torch.float32, device=logits.device)
+    ids = torch.empty((t, topk), dtype=torch.int32, device=logits.device)
+    ex = torch.empty((t,), dtype=torch.float32, device=logits.device) if extra else None
+    o._check(o._kernels().vpsa_group_topk(o._p(logits), c_int(logits.shape[1]), o._p(w), o._p(ids), o._p(ex), c_int(t),
+                                          c_int(experts), c_int(groups), c_int(keep), c_int(topk),
+                                          c_float(route_scale), o._stream()), "group_topk")
+    return w, ids, ex
+
+
+def gather_rows(x, idx):
+    if not x.is_cuda:
+        return x[idx.long()]
+    o = _ops()
+    assert x.is_contiguous() and idx.dtype == torch.int32
+    xs = torch.empty((idx.numel(), x.shape[1]), dtype=x.dtype, device=x.device)
+    o._check(o._kernels().vpsa_gather_rows(o._p(x), o._p(idx), o._p(xs), c_int(idx.numel()), c_int(x.shape[1]),
+                                           c_int(_dt(x)), o._stream()), "gather_rows")
+    return xs
+
+
+def moe_finish(residual, y, weights, pos, shared=None, gate=None):
+    """residual fp32 [T, n] += sum_k weights[t, k] * y[pos[t * K + k]] (+ gate[t] * shared[t])."""
+    if not residual.is_cuda:
+        return reference.moe_finish(residual, y, weights, pos, shared, gate)
+    o = _ops()
+    _f32(residual, weights, gate)
+    t, n = residual.shape
+    assert y.is_contiguous() and y.shape[1] == n and pos.dtype == torch.int32
+    assert shared is None or (shared.is_contiguous() and shared.shape == (t, n))
+    o._check(o._kernels().vpsa_moe_finish(o._p(residual), o._p(y), o._p(weights), o._p(pos), c_int(weights.shape[1]),
+                                          o._p(shared), o._p(gate), c_int(t), c_int(n), c_int(_dt(y, shared)),
+                                          o._stream()), "moe_finish")
+    return residual

@@ -324,3 +324,124 @@ def rans_decode(freq, states, sizes, coded, n: int, n_ctx: int, spc: int):
             x[m] = (x[m] << np.uint64(8)) | b
             rp[m] += 1
     return out.reshape(-1)
+
+
+# --------------------------------------------------------------------------- 32-bit residual stream, latent attention, group routing
+# (PyTorch definitions of csrc/kernels/latent.hip; fp32 math, results rounded to the activation dtype)
+def embed_scale(ids, embed, scale):
+    return embed[ids.long()].float() * scale
+
+
+def add_rms_norm(residual, delta, weight, eps, out_dtype, want_out=True):
+    if delta is not None:
+        residual.add_(delta.float())
+    if not want_out:
+        return None
+    inv = torch.rsqrt(residual.pow(2).mean(-1, keepdim=True) + eps)
+    return (residual * inv * weight).to(out_dtype)
+
+
+def rms_norm_rows(x, weight, eps):
+    xf = x.float()
+    return (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps) * weight).to(x.dtype)
+
+
+def _rotate_pairs(x, cs, dims):
+    """x [..., n] float: the first ``dims`` columns rotate in pairs (2i, 2i+1); cs [..., dims] = cos | sin."""
+    half = dims // 2
+    c, s = cs[..., :half], cs[..., half:]
+    u, v = x[..., 0:dims:2], x[..., 1:dims:2]
+    out = x.clone()
+    out[..., 0:dims:2] = u * c - v * s
+    out[..., 1:dims:2] = v * c + u * s
+    return out
+
+
+def latent_cache_view(pool, offset, entry):
+    """A layer's part of a [pages, page_elems] pool as [pages, PAGE, entry]."""
+    return pool[:, offset:offset + PAGE * entry].view(pool.shape[0], PAGE, entry)
+
+
+def latent_kv_write(x, weight, positions, slots, cos_sin, pool, offset, rank, rot, rot_dims, eps):
+    xf = x.float()
+    c = xf[:, :rank]
+    c = c * torch.rsqrt(c.pow(2).mean(-1, keepdim=True) + eps) * weight
+    r = _rotate_pairs(xf[:, rank:rank + rot], cos_sin[positions.long()], rot_dims)
+    view = latent_cache_view(pool, offset, rank + rot)
+    ok = slots >= 0
+    s = slots[ok].long()
+    view[s // PAGE, s % PAGE] = torch.cat([c, r], dim=-1)[ok].to(pool.dtype)
+
+
+def rope_pairs(q, positions, cos_sin, col0, rot_dims):
+    """q [T, heads, d]: columns [col0, col0 + rot_dims) of every head, in place."""
+    part = q[:, :, col0:col0 + rot_dims].float()
+    q[:, :, col0:col0 + rot_dims] = _rotate_pairs(part, cos_sin[positions.long()][:, None, :], rot_dims).to(q.dtype)
+
+
+def latent_attention(q_lat, q_rot, pool, offset, block_tables, row_seq, positions, sink, scale, out):
+    t, heads, rank = q_lat.shape
+    rot = q_rot.shape[2]
+    view = latent_cache_view(pool, offset, rank + rot)
+    seqs = row_seq.long() if row_seq is not None else torch.arange(t)
+    for s in torch.unique(seqs).tolist():
+        rows = (seqs == s).nonzero(as_tuple=True)[0]
+        pos = positions[rows].long()
+        ctx = int(pos.max()) + 1
+        pages = block_tables[s, :(ctx + PAGE - 1) // PAGE].long()
+        kv = view[pages].reshape(-1, rank + rot)[:ctx].float()
+        q = torch.cat([q_lat[rows].float(), q_rot[rows].float()], dim=-1) * scale
+        sc = torch.einsum("qhd,kd->qhk", q, kv)
+        sc = sc.masked_fill(torch.arange(ctx)[None, None, :] > pos[:, None, None], float("-inf"))
+        m = sc.max(-1).values
+        if sink is not None:
+            m = torch.maximum(m, sink[None, :])
+        e = torch.exp(sc - m[..., None])
+        den = e.sum(-1)
+        if sink is not None:
+            den = den + torch.exp(sink[None, :] - m)
+        o = torch.einsum("qhk,kd->qhd", e, kv[:, :rank]) / den[..., None]
+        out[rows] = o.to(out.dtype)
+    return out
+
+
+def sigmoid_gate(y, g):
+    y.copy_((y.float() * torch.sigmoid(g.float())[..., None]).to(y.dtype))
+    return y
+
+
+def relu_sq(x):
+    return torch.relu(x.float()).pow(2).to(x.dtype)
+
+
+def glu_clamp(x, limit, alpha, up_bias):
+    inter = x.shape[-1] // 2
+    g = x[..., :inter].float().clamp(max=limit)
+    u = x[..., inter:].float().clamp(-limit, limit)
+    return (g * torch.sigmoid(alpha * g) * (u + up_bias)).to(x.dtype)
+
+
+def group_topk(logits, experts, groups, keep, topk, route_scale, extra):
+    t = logits.shape[0]
+    s = torch.sigmoid(logits[:, :experts].float())
+    per = experts // groups
+    gs = s.view(t, groups, per)
+    score = gs.topk(min(2, per), dim=-1).values.sum(-1)
+    # stable descending order: ties go to the lower index
+    order = torch.sort(score, dim=-1, descending=True, stable=True).indices[:, :keep]
+    allowed = torch.zeros((t, groups), dtype=torch.bool)
+    allowed.scatter_(1, order, True)
+    masked = torch.where(allowed[:, :, None].expand(t, groups, per).reshape(t, experts), s, torch.full_like(s, -1.0))
+    ids = torch.sort(masked, dim=-1, descending=True, stable=True).indices[:, :topk]
+    w = s.gather(1, ids) * route_scale
+    ex = torch.sigmoid(logits[:, experts].float()) if extra else None
+    return w, ids.int(), ex
+
+
+def moe_finish(residual, y, weights, pos, shared, gate):
+    t, k = weights.shape
+    if k:
+        residual.add_((y[pos.long()].view(t, k, -1).float() * weights[:, :, None]).sum(1))
+    if shared is not None:
+        residual.add_(shared.float() * (gate[:, None] if gate is not None else 1.0))
+    return residual
