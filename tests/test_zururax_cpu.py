@@ -1,0 +1,190 @@
+"""Zururax on the CPU (the engine's PyTorch op definitions, fp32) against the float64 oracle:
+mechanisms one by one, then the engine's cache, batching and scheduler."""
+
+import math
+
+import pytest
+import torch
+
+import zururax_cases as zc
+import zururax_oracle as zo
+from vllm_production_stack_amd import ops
+from vllm_production_stack_amd.engine.config import resolve_model, zururax_layers
+
+DEV, DT, TOL = "cpu", "float32", 2e-5
+PAGE = 64
+
+
+# --------------------------------------------------------------------------- mechanisms
+def test_rope_pairs_and_norm():
+    g = torch.Generator().manual_seed(0)
+    t, heads, d, col0, dims = 9, 3, 20, 6, 10
+    q = torch.randn(t, heads, d, generator=g)
+    pos = torch.tensor([0, 1, 2, 63, 64, 65, 500, 1023, 7], dtype=torch.int32)
+    table = ops.build_cos_sin(dims, 1024, 333.0)
+    got = q.clone()
+    ops.rope_pairs(got, pos, table, col0, dims)
+    for h in range(heads):
+        want = zo.rotate_pairs(q[:, h, col0:].double(), pos, 333.0, dims)
+        assert torch.allclose(got[:, h, col0:].double(), want, atol=1e-5)
+        assert torch.equal(got[:, h, :col0], q[:, h, :col0])
+    x = torch.randn(5, 33, generator=g)
+    wgt = torch.rand(33, generator=g) + 0.5
+    assert torch.allclose(ops.rms_norm_rows(x, wgt, 1e-3).double(), zo.rms(x.double(), 1e-3, wgt.double()), atol=1e-5)
+    res, delta = torch.randn(5, 33, generator=g), torch.randn(5, 33, generator=g)
+    want = zo.rms((res + delta).double(), 1e-3, wgt.double())
+    y = ops.add_rms_norm(res, delta, wgt, 1e-3, torch.float32)
+    assert torch.allclose(y.double(), want, atol=1e-5)
+
+
+def test_gated_unit_and_dense_activation():
+    g = torch.Generator().manual_seed(1)
+    x = torch.randn(7, 2 * 11, generator=g) * 3
+    for limit in (0.5, 2.0):
+        gate = x[:, :11].double().clamp(max=limit)
+        up = x[:, 11:].double().clamp(-limit, limit)
+        want = gate * torch.sigmoid(1.702 * gate) * (up + 1)
+        assert torch.allclose(ops.glu_clamp(x, limit).double(), want, atol=1e-6)
+    assert torch.allclose(ops.relu_sq(x).double(), torch.relu(x.double()) ** 2, atol=1e-6)
+
+
+@pytest.mark.parametrize("experts,groups,keep,top", [(12, 4, 2, 3), (6, 6, 2, 1), (8, 1, 1, 4), (9, 3, 3, 2)])
+def test_group_routing(experts, groups, keep, top):
+    g = torch.Generator().manual_seed(experts)
+    h = torch.randn(40, 16, generator=g).double()
+    w = {"x.mlp.router": torch.randn(experts, 16, generator=g).double()}
+    r = {"experts": experts, "top": top, "groups": {"count": groups, "keep": keep}, "scale": 1.3}
+    want = zo.route(h, w, "x", r)
+    logits = (h @ w["x.mlp.router"].T).float()
+    extra = torch.randn(40, 1, generator=g)
+    wt, ids, ex = ops.group_topk(torch.cat([logits, extra], 1).contiguous(), experts, groups, keep, top, 1.3, extra=True)
+    for t in range(40):
+        assert [e for e, _ in want[t]] == ids[t].tolist()
+        assert torch.allclose(wt[t].double(), torch.tensor([x for _, x in want[t]], dtype=torch.float64), atol=1e-6)
+    assert torch.allclose(ex, torch.sigmoid(extra[:, 0]), atol=1e-6)
+
+
+def _attend_plain(q, entries, rank, pos, sink, scale):
+    """One row, one head, in float64: q [rank + rot] against entries [n, rank + rot] of which 0 .. pos count."""
+    s = [float(q.double() @ entries[j].double()) * scale for j in range(pos + 1)]
+    m = max(s + ([sink] if sink is not None else []))
+    e = [math.exp(x - m) for x in s]
+    den = sum(e) + (math.exp(sink - m) if sink is not None else 0.0)
+    return sum(e[j] * entries[j, :rank].double() for j in range(pos + 1)) / den
+
+
+def attention_edges(device, dtype, tol):
+    """A key whose score stands out (query and key scaled up along one direction) at the first entries, on
+    both sides of page borders, at the row's own position, and one entry past it (written by a later row of
+    the same chunk: it must stay unseen); with and without a sink, a sink that dominates."""
+    g = torch.Generator().manual_seed(3)
+    rank, rot, heads, n = 24, 8, 2, 200
+    pages = [5, 2, 7, 0]  # the sequence's pages, out of order in the pool
+    pool = torch.zeros(9, 3 * PAGE * (rank + rot) + 17, dtype=dtype, device=device)
+    offset = PAGE * (rank + rot) + 17  # another layer's entries lie before this one's
+    bt = torch.tensor([[1, 1, 1, 1], pages], dtype=torch.int32, device=device)
+    rows_pos = [0, 1, 2, 62, 63, 64, 65, 127, 128, 129, 191, 199]
+    direction = torch.randn(rank + rot, generator=g)
+    direction /= direction.norm()
+    worst = 0.0
+    for hot in (0, 1, 63, 64, 127, 128, 150, "self", "next"):
+        for sink in (None, [0.3, -1.0], [40.0, 40.0]):
+            entries = (torch.randn(n, rank + rot, generator=g) * 0.5).to(dtype).float()
+            q = torch.randn(len(rows_pos), heads, rank + rot, generator=g).to(dtype).float()
+            for i, p in enumerate(rows_pos):
+                j = p if hot == "self" else p + 1 if hot == "next" else hot
+                if j < n:
+                    entries[j] += 6.0 * direction
+                q[i] += 6.0 * direction
+            entries, q = entries.to(dtype).float(), q.to(dtype).float()
+            view = pool[:, offset:offset + PAGE * (rank + rot)].view(9, PAGE, rank + rot)
+            for j in range(n):
+                view[pages[j // PAGE], j % PAGE] = entries[j].to(dtype).to(device)
+            qd = q.to(dtype).to(device)
+            sk = None if sink is None else torch.tensor(sink, dtype=torch.float32, device=device)
+            out = ops.latent_attention(qd[:, :, :rank], qd[:, :, rank:], pool, offset, bt,
+                                       torch.ones(len(rows_pos), dtype=torch.int32, device=device),
+                                       torch.tensor(rows_pos, dtype=torch.int32, device=device), sk, 0.37)
+            for i, p in enumerate(rows_pos):
+                for h in range(heads):
+                    want = _attend_plain(q[i, h], entries, rank, p, None if sink is None else sink[h], 0.37)
+                    err = (out[i, h].double().cpu() - want).abs().max().item() / max(1e-3, want.abs().max().item())
+                    worst = max(worst, err)
+                    assert err < tol, f"hot {hot} sink {sink} row at {p} head {h}: {err:.3g}"
+    return worst
+
+
+def test_attention_edges():
+    attention_edges(torch.device("cpu"), torch.float32, 1e-4)
+
+
+def test_config_reader_and_loader(tmp_path):
+    cfg = zo.config_a()
+    folder = zo.save_checkpoint(cfg, zo.make_weights(cfg), tmp_path / "m")
+    mc, ckpt = resolve_model(folder)
+    assert mc.architecture == "zururax" and mc.num_layers == 4 and mc.embedding_scale == 3.0 and mc.norm_eps == 1e-4
+    s = mc.layer_specs
+    assert s[1].mlp is None and s[2].mixer.kv_from == 0 and s[3].mixer.kv_from == 1 and s[0].mlp.shared_ff == 40
+    assert s[3].mlp.shared_ff == 0 and (s[3].mlp.groups, s[3].mlp.keep, s[3].mlp.top) == (5, 2, 1)
+    with pytest.raises(ValueError):
+        zururax_layers([zo.layer(zo.mixer(2, 8, 4, 8, 16, 8, kv_from=0), None)])  # names itself / no earlier layer
+    # a checkpoint with a missing or a misshapen tensor is refused
+    w = zo.make_weights(cfg)
+    del w["l2.mix.sink"]
+    bad = zo.save_checkpoint(cfg, w, tmp_path / "bad")
+    from vllm_production_stack_amd.engine.config import EngineConfig
+    from vllm_production_stack_amd.engine.llm_engine import LLMEngine
+
+    with pytest.raises(ValueError):
+        LLMEngine(EngineConfig(model=bad, dtype="float32", device="cpu", num_gpu_blocks_override=4, max_model_len=256))
+
+
+# --------------------------------------------------------------------------- the engine
+@pytest.fixture(scope="module")
+def model_a():
+    cfg = zo.config_a()
+    return cfg, zo.make_weights(cfg, seed=3)
+
+
+@pytest.fixture(scope="module")
+def model_b():
+    cfg = zo.config_b()
+    return cfg, zo.make_weights(cfg, seed=4, sink_std=3.0)
+
+
+def test_layers(model_a, model_b):
+    zc.check_layers(DEV, DT, TOL, *model_a)
+    zc.check_layers(DEV, DT, TOL, *model_b)
+
+
+def test_whole_decode_and_portions(model_a):
+    n = 200
+    zc.check_cuts(DEV, DT, TOL, *model_a, n, [
+        [n],                                   # the whole prompt
+        [],                                    # token by token from the first
+        [n - 70],                              # a prompt, then 70 decoded tokens over a page border
+        [2, 2, 60, 1, 2, 61, 3, 64, 2],        # portions down to two tokens, cut at and around page borders
+        [63, 2, 63, 2], [64, 64, 64], [1, 127, 1, 1, 2],
+    ])
+
+
+def test_other_sizes(model_b):
+    zc.check_cuts(DEV, DT, TOL, *model_b, 131, [[131], [], [2, 62, 2, 63, 2], [65, 1, 1, 64]])
+
+
+def test_first_tokens(model_a):
+    for n in (1, 2, 3):
+        zc.check_cuts(DEV, DT, TOL, *model_a, n, [[n], [], [1, n]], seed=n)
+
+
+def test_long_decode(model_b):
+    zc.check_cuts(DEV, DT, TOL, *model_b, 330, [[5]], pages=6)
+
+
+def test_batches_and_reuse(model_a):
+    zc.check_batches(DEV, DT, TOL, *model_a)
+
+
+def test_greedy_generation(model_a, model_b):
+    zc.check_generate(DEV, DT, *model_a)
+    zc.check_generate(DEV, DT, *model_b, n_new=30)

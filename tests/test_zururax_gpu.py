@@ -1,0 +1,153 @@
+"""Zururax on the GPU: the HIP kernels one by one against float64 definitions, then the engine in fp32
+and in bf16 against the float64 oracle (same cases as on the CPU)."""
+
+import pytest
+import torch
+
+import zururax_cases as zc
+import zururax_oracle as zo
+from test_zururax_cpu import attention_edges
+from vllm_production_stack_amd import ops
+
+pytestmark = pytest.mark.gpu
+
+MODES = [("float32", 5e-5), ("bfloat16", 6e-2)]
+DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16}
+KERNEL_TOL = {"float32": 1e-5, "bfloat16": 2e-2}
+
+
+@pytest.fixture(scope="module")
+def model_a():
+    cfg = zo.config_a()
+    return cfg, zo.make_weights(cfg, seed=3)
+
+
+@pytest.fixture(scope="module")
+def model_b():
+    cfg = zo.config_b()
+    return cfg, zo.make_weights(cfg, seed=4, sink_std=3.0)
+
+
+def close(got, want, tol):
+    return (got.double().cpu() - want).abs().max().item() <= tol * max(1.0, want.abs().max().item())
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_elementwise_kernels(dtype):
+    dt, tol = DTYPES[dtype], KERNEL_TOL[dtype]
+    dev = torch.device("cuda")
+    g = torch.Generator().manual_seed(0)
+    # embedding times a scale into the fp32 stream
+    emb = torch.randn(50, 37, generator=g).to(dt)
+    ids = torch.randint(0, 50, (11,), generator=g)
+    assert close(ops.embed_scale(ids.to(dev), emb.to(dev), 2.5), emb[ids].double() * 2.5, 1e-6)
+    # add + norm on the fp32 stream, norm over a column range, odd sizes
+    for n in (37, 256, 1000):
+        res, delta = torch.randn(6, n, generator=g), torch.randn(6, n, generator=g).to(dt)
+        wgt = torch.rand(n, generator=g) + 0.5
+        r = res.to(dev)
+        y = ops.add_rms_norm(r, delta.to(dev), wgt.to(dev), 1e-3, dt)
+        s = res.double() + delta.double()
+        assert close(r, s, 1e-6) and close(y, zo.rms(s, 1e-3, wgt.double()), tol)
+        wide = torch.randn(6, n + 9, generator=g).to(dt)
+        y = ops.rms_norm_rows(wide.to(dev)[:, 4:4 + n], wgt.to(dev), 1e-3)
+        assert close(y, zo.rms(wide[:, 4:4 + n].double(), 1e-3, wgt.double()), tol)
+    # rotation of a column range of every head
+    q = torch.randn(9, 3, 20, generator=g).to(dt)
+    pos = torch.tensor([0, 1, 2, 63, 64, 65, 500, 1023, 7], dtype=torch.int32)
+    table = ops.build_cos_sin(10, 1024, 333.0)
+    got = q.clone().to(dev)
+    ops.rope_pairs(got, pos.to(dev), table.to(dev), 6, 10)
+    for h in range(3):
+        assert close(got[:, h, 6:], zo.rotate_pairs(q[:, h, 6:].double(), pos, 333.0, 10), tol)
+        assert torch.equal(got[:, h, :6].cpu(), q[:, h, :6])
+    # activations, output gate
+    x = (torch.randn(7, 2 * 11, generator=g) * 3).to(dt)
+    gate, up = x[:, :11].double().clamp(max=0.7), x[:, 11:].double().clamp(-0.7, 0.7)
+    assert close(ops.glu_clamp(x.to(dev), 0.7), gate * torch.sigmoid(1.702 * gate) * (up + 1), tol)
+    assert close(ops.relu_sq(x.to(dev)), torch.relu(x.double()) ** 2, tol)
+    y, gl = torch.randn(5, 3, 7, generator=g).to(dt), torch.randn(5, 9, generator=g).to(dt)
+    got = ops.sigmoid_gate(y.clone().to(dev), gl.to(dev)[:, 2:5])
+    assert close(got, y.double() * torch.sigmoid(gl[:, 2:5].double())[..., None], tol)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_cache_entries(dtype):
+    """Entries land at their slots (pages out of order, a layer's offset inside the page), normed and rotated."""
+    dt, tol = DTYPES[dtype], KERNEL_TOL[dtype]
+    dev = torch.device("cuda")
+    g = torch.Generator().manual_seed(1)
+    rank, rot, dims = 24, 12, 8
+    x = torch.randn(6, 5 + rank + rot, generator=g).to(dt)
+    wgt = torch.rand(rank, generator=g) + 0.5
+    pos = torch.tensor([0, 63, 64, 100, 5, 6], dtype=torch.int32)
+    slots = torch.tensor([3 * 64 + 0, 3 * 64 + 63, 1 * 64 + 0, 1 * 64 + 36, -1, 2 * 64 + 6])
+    pool = torch.zeros(5, 64 * (rank + rot) + 64 * 10 + 3, dtype=dt, device=dev)
+    off = 64 * 10 + 3
+    table = ops.build_cos_sin(dims, 128, 50.0)
+    ops.latent_kv_write(x.to(dev)[:, 5:], wgt.to(dev), pos.to(dev), slots.to(dev), table.to(dev), pool, off, rank, rot,
+                        dims, 1e-4)
+    view = pool[:, off:].view(5, 64, rank + rot)
+    c = zo.rms(x[:, 5:5 + rank].double(), 1e-4, wgt.double())
+    r = zo.rotate_pairs(x[:, 5 + rank:].double(), pos, 50.0, dims)
+    for i, s in enumerate(slots.tolist()):
+        if s < 0:
+            continue
+        assert close(view[s // 64, s % 64], torch.cat([c[i], r[i]]), tol)
+    assert float(pool.float().abs().sum()) == pytest.approx(float(view.float().abs().sum()))  # nothing else written
+    assert float(view[2, 5].float().abs().sum()) == 0.0  # the skipped row
+
+
+@pytest.mark.parametrize("experts,groups,keep,top", [(12, 4, 2, 3), (6, 6, 2, 1), (8, 1, 1, 4), (64, 8, 3, 6)])
+def test_group_routing(experts, groups, keep, top):
+    g = torch.Generator().manual_seed(experts)
+    h = torch.randn(70, 16, generator=g).double()
+    w = {"x.mlp.router": torch.randn(experts, 16, generator=g).double()}
+    want = zo.route(h, w, "x", {"experts": experts, "top": top, "groups": {"count": groups, "keep": keep}, "scale": 1.3})
+    logits = torch.cat([(h @ w["x.mlp.router"].T).float(), torch.randn(70, 1, generator=g)], 1).contiguous()
+    wt, ids, ex = ops.group_topk(logits.cuda(), experts, groups, keep, top, 1.3, extra=True)
+    for t in range(70):
+        assert [e for e, _ in want[t]] == ids[t].tolist()
+        assert torch.allclose(wt[t].double().cpu(), torch.tensor([x for _, x in want[t]], dtype=torch.float64), atol=1e-6)
+    assert torch.allclose(ex.cpu(), torch.sigmoid(logits[:, experts]), atol=1e-6)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_attention_edges(dtype):
+    attention_edges(torch.device("cuda"), DTYPES[dtype], 2e-4 if dtype == "float32" else 3e-2)
+
+
+@pytest.mark.parametrize("dtype,tol", MODES)
+def test_layers(dtype, tol, model_a, model_b):
+    zc.check_layers("cuda", dtype, tol, *model_a)
+    zc.check_layers("cuda", dtype, tol, *model_b)
+
+
+@pytest.mark.parametrize("dtype,tol", MODES)
+def test_whole_decode_and_portions(dtype, tol, model_a):
+    n = 200
+    zc.check_cuts("cuda", dtype, tol, *model_a, n, [
+        [n], [], [n - 70], [2, 2, 60, 1, 2, 61, 3, 64, 2], [63, 2, 63, 2], [64, 64, 64], [1, 127, 1, 1, 2]])
+
+
+@pytest.mark.parametrize("dtype,tol", MODES)
+def test_other_sizes_and_first_tokens(dtype, tol, model_a, model_b):
+    zc.check_cuts("cuda", dtype, tol, *model_b, 131, [[131], [], [2, 62, 2, 63, 2], [65, 1, 1, 64]])
+    for n in (1, 2, 3):
+        zc.check_cuts("cuda", dtype, tol, *model_a, n, [[n], [], [1, n]], seed=n)
+
+
+@pytest.mark.parametrize("dtype,tol", MODES)
+def test_long_decode(dtype, tol, model_b):
+    zc.check_cuts("cuda", dtype, tol, *model_b, 330, [[5]], pages=6)
+
+
+@pytest.mark.parametrize("dtype,tol", MODES)
+def test_batches_and_reuse(dtype, tol, model_a):
+    zc.check_batches("cuda", dtype, tol, *model_a)
+
+
+def test_greedy_generation(model_a, model_b):
+    zc.check_generate("cuda", "float32", *model_a)
+    zc.check_generate("cuda", "float32", *model_b, n_new=30)
+    assert ops.native_loaded()

@@ -1,0 +1,248 @@
+"""Plain float64 definition of the Zururax decoder, one function per mechanism, and makers of small
+random checkpoints.  It recomputes whole sequences (no cache, no batching, keys and values expanded
+per head) and shares no code with the engine; the engine's tests compare against it."""
+
+from __future__ import annotations
+
+import json
+import math
+from pathlib import Path
+
+import torch
+
+F64 = torch.float64
+
+
+# --------------------------------------------------------------------------- mechanisms
+def rms(x, eps, w=None):
+    y = x / torch.sqrt((x * x).mean(-1, keepdim=True) + eps)
+    return y if w is None else y * w
+
+
+def rotate_pairs(x, pos, base, dims):
+    """x [T, n]: channels (2i, 2i+1), i < dims/2, turn by pos * base^(-2i/dims); the rest pass."""
+    out = x.clone()
+    for i in range(dims // 2):
+        a = pos.to(F64) * base ** (-2.0 * i / dims)
+        u, v = x[:, 2 * i], x[:, 2 * i + 1]
+        out[:, 2 * i] = u * torch.cos(a) - v * torch.sin(a)
+        out[:, 2 * i + 1] = v * torch.cos(a) + u * torch.sin(a)
+    return out
+
+
+def sink_softmax(scores, sink):
+    """scores [T, T] already masked with -inf; the denominator also holds exp(sink)."""
+    m = scores.max(-1, keepdim=True).values
+    if sink is not None:
+        m = torch.maximum(m, torch.full_like(m, float(sink)))
+    e = torch.exp(scores - m)
+    den = e.sum(-1, keepdim=True)
+    if sink is not None:
+        den = den + torch.exp(float(sink) - m)
+    return e / den
+
+
+def latent_kv(h, w, p, m, pos, eps):
+    """The cached pair of a layer that owns its entries: (latent c [T, kv_rank], rotated key part [T, rot_dim])."""
+    dkv = h @ w[p + ".mix.dkv"].T
+    c = rms(dkv[:, :m["kv_rank"]], eps, w[p + ".mix.dkv.norm"])
+    kr = rotate_pairs(dkv[:, m["kv_rank"]:], pos, m["rot"]["base"], m["rot"]["dims"])
+    return c, kr
+
+
+def latent_attention(h, w, p, m, pos, eps, c, kr):
+    t = h.shape[0]
+    H, D, R, V = m["heads"], m["dim"], m["rot_dim"], m["vdim"]
+    cq = rms(h @ w[p + ".mix.dq"].T, eps, w[p + ".mix.dq.norm"])
+    q = (cq @ w[p + ".mix.uq"].T).view(t, H, D + R)
+    k_all = (c @ w[p + ".mix.uk"].T).view(t, H, D)
+    v_all = (c @ w[p + ".mix.uv"].T).view(t, H, V)
+    gate = torch.sigmoid(h @ w[p + ".mix.g"].T)
+    future = pos[None, :] > pos[:, None]
+    heads = []
+    for hd in range(H):
+        qn = q[:, hd, :D]
+        qr = rotate_pairs(q[:, hd, D:], pos, m["rot"]["base"], m["rot"]["dims"])
+        sc = (qn @ k_all[:, hd].T + qr @ kr.T) * m["scale"]
+        sc = sc.masked_fill(future, -math.inf)
+        pr = sink_softmax(sc, w[p + ".mix.sink"][hd])
+        heads.append((pr @ v_all[:, hd]) * gate[:, hd:hd + 1])
+    return torch.cat(heads, dim=-1) @ w[p + ".mix.o"].T
+
+
+def dense_ff(h, w, p):
+    return torch.relu(h @ w[p + ".mlp.up"].T) ** 2 @ w[p + ".mlp.down"].T
+
+
+def gated_unit(h, w, p, limit):
+    g = torch.clamp(h @ w[p + ".gate"].T, max=limit)
+    u = torch.clamp(h @ w[p + ".up"].T, -limit, limit)
+    return (g * torch.sigmoid(1.702 * g) * (u + 1)) @ w[p + ".down"].T
+
+
+def route(h, w, p, r):
+    """-> per token: list of (expert, weight)."""
+    s = torch.sigmoid(h @ w[p + ".mlp.router"].T)
+    E, top = r["experts"], r["top"]
+    groups = r.get("groups") or {"count": 1, "keep": 1}
+    G, keep = groups["count"], groups["keep"]
+    per = E // G
+    out = []
+    for t in range(h.shape[0]):
+        score = []
+        for g in range(G):
+            best = sorted((float(x) for x in s[t, g * per:(g + 1) * per]), reverse=True)[:2]
+            score.append(sum(best))
+        kept = sorted(range(G), key=lambda g: (-score[g], g))[:keep]
+        cand = [e for g in kept for e in range(g * per, (g + 1) * per)]
+        chosen = sorted(cand, key=lambda e: (-float(s[t, e]), e))[:top]
+        out.append([(e, float(s[t, e]) * r["scale"]) for e in chosen])
+    return out
+
+
+def moe_ff(h, w, p, mlp):
+    y = torch.zeros_like(h)
+    for t, picks in enumerate(route(h, w, p, mlp["router"])):
+        for e, wt in picks:
+            y[t] += wt * gated_unit(h[t:t + 1], w, f"{p}.mlp.e{e}", mlp["expert"]["limit"])[0]
+    if mlp.get("shared"):
+        sg = torch.sigmoid(h @ w[p + ".mlp.shared.sg"].T)
+        y = y + sg * gated_unit(h, w, p + ".mlp.shared", mlp["shared"]["limit"])
+    return y
+
+
+def forward(cfg, w, tokens, layers_out=None):
+    """Logits [T, vocab] of a whole sequence (float64)."""
+    eps = cfg["norm"]["eps"]
+    pos = torch.arange(len(tokens))
+    x = w["embed"][torch.tensor(tokens)] * cfg["embedding"]["scale"]
+    held = {}
+    for i, layer in enumerate(cfg["layers"]):
+        p, m = f"l{i}", layer["mixer"]
+        h = rms(x, eps, w[p + ".norm1"])
+        if m.get("kv_from") is None:
+            held[i] = latent_kv(h, w, p, m, pos, eps)
+        c, kr = held[i if m.get("kv_from") is None else m["kv_from"]]
+        x = x + latent_attention(h, w, p, m, pos, eps, c, kr)
+        mlp = layer.get("mlp")
+        if mlp is not None:
+            h = rms(x, eps, w[p + ".norm2"])
+            x = x + (dense_ff(h, w, p) if mlp["kind"] == "dense" else moe_ff(h, w, p, mlp))
+        if layers_out is not None:
+            layers_out.append(x.clone())
+    return rms(x, eps, w["final.norm"]) @ w["head"].T
+
+
+def greedy(cfg, w, prompt, n):
+    ids = list(prompt)
+    for _ in range(n):
+        ids.append(int(forward(cfg, w, ids)[-1].argmax()))
+    return ids[len(prompt):]
+
+
+# --------------------------------------------------------------------------- checkpoints
+def mixer(heads, dim, rot_dim, vdim, kv_rank, q_rank, base=10000.0, kv_from=None, scale=None):
+    m = {"heads": heads, "dim": dim, "rot_dim": rot_dim, "vdim": vdim, "kv_rank": kv_rank, "q_rank": q_rank,
+         "rot": {"base": base, "dims": rot_dim}, "scale": scale if scale is not None else (dim + rot_dim) ** -0.5}
+    if kv_from is not None:
+        m["kv_from"] = kv_from
+    return m
+
+
+def moe(ff, experts, top, groups, keep, shared_ff=0, scale=1.0, limit=2.0, shared_limit=3.0):
+    return {"kind": "moe", "expert": {"ff": ff, "limit": limit},
+            "router": {"experts": experts, "top": top, "groups": {"count": groups, "keep": keep}, "scale": scale},
+            "shared": {"ff": shared_ff, "limit": shared_limit} if shared_ff else None}
+
+
+def layer(m, mlp):
+    return {"type": "latent_attention", "mixer": m, "mlp": mlp}
+
+
+def make_config(vocab, width, layers, embedding_scale=1.0, eps=1e-5):
+    return {"architecture": "Zururax", "embedding": {"scale": embedding_scale}, "layers": layers,
+            "norm": {"eps": eps}, "vocab": vocab, "width": width}
+
+
+def config_a():
+    """Unequal dim / rot_dim / vdim, a layer without feed-forward, a dense layer that is not the first, a
+    far kv_from, groups of one expert, top 1 and top 3, a mixture without a shared unit."""
+    return make_config(97, 72, [
+        layer(mixer(3, 16, 8, 24, 40, 24, base=500.0), moe(24, 6, 3, 3, 2, shared_ff=40, scale=1.7, limit=0.8)),
+        layer(mixer(2, 8, 12, 16, 56, 32, base=20000.0), None),
+        layer(mixer(3, 24, 8, 8, 40, 16, base=500.0, kv_from=0), {"kind": "dense", "ff": 104}),
+        layer(mixer(1, 16, 12, 32, 56, 40, base=20000.0, kv_from=1), moe(16, 5, 1, 5, 2, shared_ff=0, scale=0.9)),
+    ], embedding_scale=3.0, eps=1e-4)
+
+
+def config_b():
+    """One group (no group limit), keep == count, every layer caching, heads of one channel pair."""
+    return make_config(61, 48, [
+        layer(mixer(4, 2, 2, 4, 24, 8), moe(8, 4, 2, 1, 1, shared_ff=8, scale=2.0, limit=5.0, shared_limit=0.5)),
+        layer(mixer(2, 12, 20, 12, 32, 48, base=77.0), moe(8, 8, 4, 4, 4, shared_ff=0, scale=0.5)),
+    ], embedding_scale=0.25)
+
+
+def make_weights(cfg, seed=0, sink_std=1.0):
+    """bf16-representable float64 weights (what a bf16 checkpoint holds), activations of order one."""
+    g = torch.Generator().manual_seed(seed)
+
+    def rnd(*shape, std=None):
+        t = torch.randn(shape, generator=g, dtype=torch.float32) * (std if std is not None else shape[-1] ** -0.5)
+        return t.to(torch.bfloat16).to(F64)
+
+    def gain(n):
+        return (1.0 + 0.3 * torch.randn(n, generator=g)).to(torch.bfloat16).to(F64)
+
+    wd, w = cfg["width"], {}
+    w["embed"] = rnd(cfg["vocab"], wd, std=1.0)
+    for i, L in enumerate(cfg["layers"]):
+        p, m, f = f"l{i}", L["mixer"], L.get("mlp")
+        H, D, R, V, KR, QR = m["heads"], m["dim"], m["rot_dim"], m["vdim"], m["kv_rank"], m["q_rank"]
+        w[p + ".norm1"] = gain(wd)
+        w[p + ".mix.dq"], w[p + ".mix.dq.norm"] = rnd(QR, wd), gain(QR)
+        w[p + ".mix.uq"] = rnd(H * (D + R), QR, std=2.0 * QR ** -0.5)
+        if m.get("kv_from") is None:
+            w[p + ".mix.dkv"], w[p + ".mix.dkv.norm"] = rnd(KR + R, wd), gain(KR)
+        w[p + ".mix.uk"] = rnd(H * D, KR, std=2.0 * KR ** -0.5)
+        w[p + ".mix.uv"] = rnd(H * V, KR)
+        w[p + ".mix.sink"] = rnd(H, std=sink_std)
+        w[p + ".mix.g"] = rnd(H, wd, std=2.0 * wd ** -0.5)
+        w[p + ".mix.o"] = rnd(wd, H * V)
+        if f is None:
+            continue
+        w[p + ".norm2"] = gain(wd)
+        if f["kind"] == "dense":
+            w[p + ".mlp.up"], w[p + ".mlp.down"] = rnd(f["ff"], wd), rnd(wd, f["ff"])
+        else:
+            w[p + ".mlp.router"] = rnd(f["router"]["experts"], wd, std=3.0 * wd ** -0.5)
+            units = [(f"{p}.mlp.e{e}", f["expert"]["ff"]) for e in range(f["router"]["experts"])]
+            if f.get("shared"):
+                units.append((p + ".mlp.shared", f["shared"]["ff"]))
+                w[p + ".mlp.shared.sg"] = rnd(1, wd, std=2.0 * wd ** -0.5)
+            for name, ff in units:
+                w[name + ".gate"], w[name + ".up"] = rnd(ff, wd, std=2.0 * wd ** -0.5), rnd(ff, wd, std=2.0 * wd ** -0.5)
+                w[name + ".down"] = rnd(wd, ff)
+    w["final.norm"] = gain(wd)
+    w["head"] = rnd(cfg["vocab"], wd)
+    return w
+
+
+def save_checkpoint(cfg, w, folder) -> str:
+    from safetensors.torch import save_file
+
+    folder = Path(folder)
+    folder.mkdir(parents=True, exist_ok=True)
+    with open(folder / "config.json", "w") as f:
+        json.dump(cfg, f)
+    save_file({k: v.to(torch.bfloat16).contiguous() for k, v in w.items()}, str(folder / "model.safetensors"))
+    return str(folder)
+
+
+def rel_error(got, want):
+    """Row-wise error of logits as the root mean square of the mean-free difference over that of ``want``."""
+    got, want = got.to(F64), want.to(F64)
+    d = got - want
+    d = d - d.mean(-1, keepdim=True)
+    scale = (want - want.mean(-1, keepdim=True)).pow(2).mean().sqrt()
+    return (d.pow(2).mean(-1).sqrt() / scale).max().item()
