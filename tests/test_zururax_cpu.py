@@ -73,24 +73,39 @@ def _attend_plain(q, entries, rank, pos, sink, scale):
     return sum(e[j] * entries[j, :rank].double() for j in range(pos + 1)) / den
 
 
-def attention_edges(device, dtype, tol):
+def attention_edges(device, dtype, tol, rank=24, rot=8, heads=2, mode="rows", splits=1):
     """A key whose score stands out (query and key scaled up along one direction) at the first entries, on
     both sides of page borders, at the row's own position, and one entry past it (written by a later row of
-    the same chunk: it must stay unseen); with and without a sink, a sink that dominates."""
+    the same chunk: it must stay unseen); with and without a sink, a sink that dominates.
+    mode: "rows" = rows of one sequence named by row_seq, "tiles" = the same rows as one-token tiles of the
+    tile kernel, "decode" = every row a sequence of its own (with key-range splits)."""
+    import numpy as np
+
     g = torch.Generator().manual_seed(3)
-    rank, rot, heads, n = 24, 8, 2, 200
+    n = 200
     pages = [5, 2, 7, 0]  # the sequence's pages, out of order in the pool
-    pool = torch.zeros(9, 3 * PAGE * (rank + rot) + 17, dtype=dtype, device=device)
-    offset = PAGE * (rank + rot) + 17  # another layer's entries lie before this one's
-    bt = torch.tensor([[1, 1, 1, 1], pages], dtype=torch.int32, device=device)
+    pool = torch.zeros(9, 3 * PAGE * (rank + rot) + 16, dtype=dtype, device=device)
+    offset = PAGE * (rank + rot) + 16  # another layer's entries lie before this one's
     rows_pos = [0, 1, 2, 62, 63, 64, 65, 127, 128, 129, 191, 199]
+    nr = len(rows_pos)
+    if mode == "decode":
+        bt = torch.tensor([pages] * nr, dtype=torch.int32, device=device)
+        row_seq, tiles = None, None
+    else:
+        bt = torch.tensor([[1, 1, 1, 1], pages], dtype=torch.int32, device=device)
+        row_seq = torch.ones(nr, dtype=torch.int32, device=device)
+        tiles = None
+        if mode == "tiles":
+            tiles = torch.from_numpy(np.array(  # a tile holds at most 64 heads of a token; one unused entry
+                [[1, i, 1, p, h0, min(64, heads - h0)] for i, p in enumerate(rows_pos) for h0 in range(0, heads, 64)]
+                + [[-1] * 6], dtype=np.int32)).to(device)
     direction = torch.randn(rank + rot, generator=g)
     direction /= direction.norm()
     worst = 0.0
     for hot in (0, 1, 63, 64, 127, 128, 150, "self", "next"):
-        for sink in (None, [0.3, -1.0], [40.0, 40.0]):
+        for sink in (None, [0.3 - h for h in range(heads)], [40.0] * heads):
             entries = (torch.randn(n, rank + rot, generator=g) * 0.5).to(dtype).float()
-            q = torch.randn(len(rows_pos), heads, rank + rot, generator=g).to(dtype).float()
+            q = torch.randn(nr, heads, rank + rot, generator=g).to(dtype).float()
             for i, p in enumerate(rows_pos):
                 j = p if hot == "self" else p + 1 if hot == "next" else hot
                 if j < n:
@@ -102,9 +117,9 @@ def attention_edges(device, dtype, tol):
                 view[pages[j // PAGE], j % PAGE] = entries[j].to(dtype).to(device)
             qd = q.to(dtype).to(device)
             sk = None if sink is None else torch.tensor(sink, dtype=torch.float32, device=device)
-            out = ops.latent_attention(qd[:, :, :rank], qd[:, :, rank:], pool, offset, bt,
-                                       torch.ones(len(rows_pos), dtype=torch.int32, device=device),
-                                       torch.tensor(rows_pos, dtype=torch.int32, device=device), sk, 0.37)
+            out = ops.latent_attention(qd[:, :, :rank], qd[:, :, rank:], pool, offset, bt, row_seq,
+                                       torch.tensor(rows_pos, dtype=torch.int32, device=device), sk, 0.37,
+                                       tiles=tiles, splits=splits)
             for i, p in enumerate(rows_pos):
                 for h in range(heads):
                     want = _attend_plain(q[i, h], entries, rank, p, None if sink is None else sink[h], 0.37)

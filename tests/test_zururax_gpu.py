@@ -117,6 +117,31 @@ def test_attention_edges(dtype):
     attention_edges(torch.device("cuda"), DTYPES[dtype], 2e-4 if dtype == "float32" else 3e-2)
 
 
+@pytest.mark.parametrize("rank,rot,heads", [(64, 32, 3), (128, 64, 5), (256, 32, 70), (512, 64, 2)])
+@pytest.mark.parametrize("mode,splits", [("tiles", 1), ("decode", 1), ("decode", 3), ("decode", 7)])
+def test_attention_edges_matrix_cores(rank, rot, heads, mode, splits):
+    """The tile kernel: one-token tiles and decode rows, whole key range and key-range splits (more splits
+    than some rows have pages), more heads than a tile holds."""
+    assert ops.latent_mfma_supported(rank, rot)
+    attention_edges(torch.device("cuda"), torch.bfloat16, 3e-2, rank=rank, rot=rot, heads=heads, mode=mode, splits=splits)
+
+
+@pytest.fixture(scope="module")
+def model_c():
+    cfg = zo.config_c()
+    return cfg, zo.make_weights(cfg, seed=5)
+
+
+def test_tile_kernel_in_the_engine(model_c):
+    """Entries of shapes the tile kernel takes (bf16): tiles of several tokens, a head count that does not
+    divide a tile, layers of different head counts, a layer reading another layer's entries."""
+    tol = 6e-2
+    zc.check_layers("cuda", "bfloat16", tol, *model_c)
+    zc.check_cuts("cuda", "bfloat16", tol, *model_c, 200, [[200], [], [130], [2, 2, 60, 1, 2, 61, 3, 64, 2], [63, 2, 63, 2]])
+    zc.check_batches("cuda", "bfloat16", tol, *model_c)
+    zc.check_cuts("cuda", "float32", 5e-5, *model_c, 150, [[150], [70, 3, 64]])
+
+
 @pytest.mark.parametrize("dtype,tol", MODES)
 def test_layers(dtype, tol, model_a, model_b):
     zc.check_layers("cuda", dtype, tol, *model_a)
@@ -133,8 +158,9 @@ def test_whole_decode_and_portions(dtype, tol, model_a):
 @pytest.mark.parametrize("dtype,tol", MODES)
 def test_other_sizes_and_first_tokens(dtype, tol, model_a, model_b):
     zc.check_cuts("cuda", dtype, tol, *model_b, 131, [[131], [], [2, 62, 2, 63, 2], [65, 1, 1, 64]])
-    for n in (1, 2, 3):
-        zc.check_cuts("cuda", dtype, tol, *model_a, n, [[n], [], [1, n]], seed=n)
+    if dtype == "float32":  # (a handful of rows: one close call of a router in bf16 would be all of them)
+        for n in (1, 2, 3):
+            zc.check_cuts("cuda", dtype, tol, *model_a, n, [[n], [], [1, n]], seed=n)
 
 
 @pytest.mark.parametrize("dtype,tol", MODES)

@@ -183,6 +183,15 @@ def config_b():
     ], embedding_scale=0.25)
 
 
+def config_c():
+    """Cache entries of 64 + 32 and 128 + 32 values, 3 and 5 heads, a layer that reads its neighbour's entries."""
+    return make_config(83, 64, [
+        layer(mixer(3, 16, 32, 8, 64, 24, base=300.0), {"kind": "dense", "ff": 72}),
+        layer(mixer(5, 8, 32, 16, 64, 32, base=300.0, kv_from=0), moe(16, 4, 2, 2, 1, shared_ff=24, scale=1.2)),
+        layer(mixer(2, 24, 32, 32, 128, 40, base=9000.0), None),
+    ], embedding_scale=1.5)
+
+
 def make_weights(cfg, seed=0, sink_std=1.0):
     """bf16-representable float64 weights (what a bf16 checkpoint holds), activations of order one."""
     g = torch.Generator().manual_seed(seed)
@@ -239,10 +248,27 @@ def save_checkpoint(cfg, w, folder) -> str:
     return str(folder)
 
 
-def rel_error(got, want):
-    """Row-wise error of logits as the root mean square of the mean-free difference over that of ``want``."""
+def row_errors(got, want):
+    """Per row: root mean square of the mean-free difference of the logits, over that of ``want`` as a whole."""
     got, want = got.to(F64), want.to(F64)
     d = got - want
     d = d - d.mean(-1, keepdim=True)
     scale = (want - want.mean(-1, keepdim=True)).pow(2).mean().sqrt()
-    return (d.pow(2).mean(-1).sqrt() / scale).max().item()
+    return d.pow(2).mean(-1).sqrt() / scale
+
+
+def rel_error(got, want):
+    return row_errors(got, want).max().item()
+
+
+def check_rows(got, want, tol, what=""):
+    """32-bit runs (tol < 1e-3): every row within tol.  bf16 runs: the typical row well within tol, and at
+    most one row in twenty-five (or one) beyond it: with random weights a router's close call now and then falls
+    the other way in bf16, which changes that row's logits altogether and means nothing."""
+    e = row_errors(got, want)
+    if tol < 1e-3:
+        assert e.max().item() < tol, f"{what}: error {e.max().item():.3g} at row {int(e.argmax())}"
+        return
+    far = int((e > tol).sum())  # (more routed units per token: more close calls)
+    assert e.median().item() < tol / 3, f"{what}: median error {e.median().item():.3g}"
+    assert far <= max(1, len(e) // 25), f"{what}: {far} of {len(e)} rows beyond {tol}, worst {e.max().item():.3g}"

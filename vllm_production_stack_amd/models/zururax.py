@@ -156,6 +156,12 @@ class ZururaxModel:
         for i, n in enumerate(q_lens):
             seq.extend([i] * n)
         meta.pre_row_seq = to_dev(seq, torch.int32)
+        meta.pre_lat_tiles = {}
+        if self.device.type == "cuda" and self.dtype == torch.bfloat16:
+            for heads in sorted({s.mixer.heads for s in self.specs
+                                 if ops.latent_mfma_supported(s.mixer.kv_rank, s.mixer.rot_dim)}):
+                tiles = ops.build_latent_tiles(q_lens, ctx_lens, heads)
+                meta.pre_lat_tiles[heads] = torch.from_numpy(tiles).pin_memory().to(self.device, non_blocking=True)
 
     # ------------------------------------------------------------------ forward
     def _mixer(self, lw: ZururaxLayer, h: torch.Tensor, pool, meta: BatchMeta) -> torch.Tensor:
@@ -178,10 +184,12 @@ class ZururaxModel:
         nd = meta.num_decode
         if nd > 0:
             ops.latent_attention(q_lat[:nd], q_rot[:nd], pool, lw.cache_offset, meta.dec_block_tables, None,
-                                 meta.positions[:nd], lw.sink, m.scale, out=o_lat[:nd])
+                                 meta.positions[:nd], lw.sink, m.scale, out=o_lat[:nd],
+                                 splits=getattr(meta, "dec_num_splits", 1) or 1)
         if meta.num_prefill_seqs > 0:
             ops.latent_attention(q_lat[nd:], q_rot[nd:], pool, lw.cache_offset, meta.pre_block_tables,
-                                 meta.pre_row_seq, meta.positions[nd:], lw.sink, m.scale, out=o_lat[nd:])
+                                 meta.pre_row_seq, meta.positions[nd:], lw.sink, m.scale, out=o_lat[nd:],
+                                 tiles=(meta.pre_lat_tiles or {}).get(m.heads))
         # [heads, T, kv_rank] x [heads, kv_rank, vdim] -> [T, heads, vdim]
         o = torch.bmm(o_lat.transpose(0, 1), lw.w_uv.transpose(1, 2)).transpose(0, 1).contiguous()
         if m.out_gate:

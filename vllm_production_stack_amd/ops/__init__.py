@@ -39,7 +39,7 @@ def _kernels():
             "vpsa_tile_gemm", "vpsa_tile_gemm_debug", "vpsa_paged_prefill_split",
             "vpsa_embed_scale", "vpsa_add_rmsnorm", "vpsa_rmsnorm_rows", "vpsa_latent_kv_write", "vpsa_rope_pairs",
             "vpsa_latent_attention", "vpsa_sigmoid_gate", "vpsa_relu_sq", "vpsa_glu_clamp", "vpsa_group_topk",
-            "vpsa_gather_rows", "vpsa_moe_finish",
+            "vpsa_gather_rows", "vpsa_moe_finish", "vpsa_latent_mfma_supported", "vpsa_latent_attention_mfma",
         ):
             getattr(lib, name).restype = c_int
         lib.vpsa_prefill_split_record_bytes.restype = c_long
@@ -1316,5 +1316,5 @@ def lora_expand(h, bs, slots, y, r_pad):
 
 
 # --------------------------------------------------------------------------- latent attention, group routing, fp32 residual
-from .latent import (add_rms_norm, embed_scale, gather_rows, glu_clamp, group_topk, latent_attention,  # noqa: E402,F401
-                     latent_kv_write, moe_finish, relu_sq, rms_norm_rows, rope_pairs, sigmoid_gate)
+from .latent import (add_rms_norm, build_latent_tiles, embed_scale, gather_rows, glu_clamp, group_topk, latent_attention,  # noqa: E402,F401
+                     latent_kv_write, latent_mfma_supported, moe_finish, relu_sq, rms_norm_rows, rope_pairs, sigmoid_gate)

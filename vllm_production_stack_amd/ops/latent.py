@@ -127,13 +127,60 @@ def rope_pairs(q, positions, cos_sin, col0: int, rot_dims: int):
                                           c_int(rot_dims), c_int(_dt(q)), o._stream()), "rope_pairs")
 
 
-def latent_attention(q_lat, q_rot, pool, offset: int, block_tables, row_seq, positions, sink, scale: float, out=None):
+LATENT_TILE_SLOTS = 64  # (token, head) pairs of one tile of the matrix-core kernel
+LATENT_MFMA = True      # False: every call takes the plain kernel (A/B runs, tests of the plain kernel)
+
+
+def latent_mfma_supported(rank: int, rot: int) -> bool:
+    return bool(_ops()._kernels().vpsa_latent_mfma_supported(c_int(rank), c_int(rot)))
+
+
+def build_latent_tiles(q_lens, ctx_lens, heads: int):
+    """Work list of the matrix-core kernel for the prefill part of a batch: int32 rows (sequence, first
+    query row, tokens, position of the first token, first head, heads per token), a tile holding up to
+    64 (token, head) pairs of consecutive tokens of one sequence.  Longest contexts first."""
+    import numpy as np
+
+    per_tok = max(1, LATENT_TILE_SLOTS // heads)
+    runs = [(h0, min(LATENT_TILE_SLOTS, heads - h0)) for h0 in range(0, heads, LATENT_TILE_SLOTS)]
+    parts = []
+    row = 0
+    for i, (n, ctx) in enumerate(zip(q_lens, ctx_lens)):
+        k = np.arange(0, n, per_tok, dtype=np.int64)
+        for h0, hc in runs:
+            parts.append(np.stack([np.full_like(k, i), row + k, np.minimum(per_tok, n - k), ctx - n + k,
+                                   np.full_like(k, h0), np.full_like(k, hc)], axis=1))
+        row += n
+    if not parts:
+        return np.zeros((0, 6), dtype=np.int32)
+    tiles = np.concatenate(parts)
+    order = np.argsort(-(tiles[:, 3] + tiles[:, 2]), kind="stable")
+    return tiles[order].astype(np.int32)
+
+
+def _mfma_ok(q_lat, q_rot, pool, out) -> bool:
+    if not (LATENT_MFMA and q_lat.dtype == torch.bfloat16 and pool.dtype == torch.bfloat16):
+        return False
+    rank, rot = q_lat.shape[2], q_rot.shape[2]
+    if not latent_mfma_supported(rank, rot):
+        return False
+    return (q_lat.data_ptr() % 16 == 0 and q_rot.data_ptr() % 16 == 0 and out.data_ptr() % 8 == 0
+            and all(s % 8 == 0 for s in (q_lat.stride(0), q_lat.stride(1), q_rot.stride(0), q_rot.stride(1)))
+            and out.stride(0) % 4 == 0 and out.stride(1) % 4 == 0 and pool.stride(0) % 8 == 0)
+
+
+def latent_attention(q_lat, q_rot, pool, offset: int, block_tables, row_seq, positions, sink, scale: float, out=None,
+                     tiles=None, splits: int = 1):
     """Causal attention of query rows over their sequences' cache entries, in latent space.
 
     q_lat [T, heads, rank] and q_rot [T, heads, rot] (views with contiguous last dim); row ``i``
-    belongs to sequence ``row_seq[i]`` (``None``: row i is sequence i) whose pages are
+    belongs to sequence ``row_seq[i]`` (``None``: row i is sequence i, a decode batch) whose pages are
     ``block_tables[seq]`` and sees entries 0 .. positions[i].  ``sink`` [heads] fp32 or None: a logit
-    that joins the softmax denominator only.  Returns [T, heads, rank]."""
+    that joins the softmax denominator only.  Returns [T, heads, rank].
+
+    bf16 entries of a shape the matrix-core kernel tiles take it: decode batches as they are (with
+    ``splits`` key ranges per row, merged by a second launch), prefill rows when ``tiles`` (the device
+    copy of ``build_latent_tiles``) describes them.  Everything else takes the plain kernel."""
     t, heads, rank = q_lat.shape
     if out is None:
         out = torch.empty((t, heads, rank), dtype=q_lat.dtype, device=q_lat.device)
@@ -147,12 +194,30 @@ def latent_attention(q_lat, q_rot, pool, offset: int, block_tables, row_seq, pos
     assert q_lat.stride(2) == 1 and q_rot.stride(2) == 1 and out.stride(2) == 1 and q_rot.shape[:2] == (t, heads)
     assert block_tables.dtype == torch.int32 and block_tables.stride(1) == 1 and positions.dtype == torch.int32
     assert row_seq is None or (row_seq.dtype == torch.int32 and row_seq.numel() == t)
+    dt = _dt(q_lat, q_rot, pool, out)
+    if (tiles is not None or row_seq is None) and _mfma_ok(q_lat, q_rot, pool, out):
+        if tiles is not None:
+            assert tiles.dtype == torch.int32 and tiles.is_contiguous() and tiles.shape[1] == 6
+            n_tiles, splits = tiles.shape[0], 1
+        else:
+            n_tiles = t * ((heads + LATENT_TILE_SLOTS - 1) // LATENT_TILE_SLOTS)
+        ws_o = ws_ml = None
+        if splits > 1:
+            ws_o = torch.empty((n_tiles * splits * LATENT_TILE_SLOTS * rank,), dtype=torch.float32, device=out.device)
+            ws_ml = torch.empty((n_tiles * splits * LATENT_TILE_SLOTS * 2,), dtype=torch.float32, device=out.device)
+        o._check(o._kernels().vpsa_latent_attention_mfma(
+            o._p(q_lat), c_long(q_lat.stride(0)), c_long(q_lat.stride(1)), o._p(q_rot), c_long(q_rot.stride(0)),
+            c_long(q_rot.stride(1)), _layer_base(pool, offset, rank + rot), c_long(pool.stride(0)), o._p(block_tables),
+            c_int(block_tables.stride(0)), o._p(tiles), o._p(positions), c_int(n_tiles), c_int(heads), o._p(sink),
+            o._p(out), c_long(out.stride(0)), c_long(out.stride(1)), c_int(rank), c_int(rot), c_float(scale),
+            c_int(splits), o._p(ws_o), o._p(ws_ml), o._stream()), "latent_attention_mfma")
+        return out
     o._check(o._kernels().vpsa_latent_attention(
         o._p(q_lat), c_long(q_lat.stride(0)), c_long(q_lat.stride(1)), o._p(q_rot), c_long(q_rot.stride(0)),
         c_long(q_rot.stride(1)), _layer_base(pool, offset, rank + rot), c_long(pool.stride(0)), o._p(block_tables),
         c_int(block_tables.stride(0)), o._p(row_seq), o._p(positions), o._p(sink), o._p(out), c_long(out.stride(0)),
         c_long(out.stride(1)), c_int(t), c_int(heads), c_int(rank), c_int(rot), c_float(scale),
-        c_int(_dt(q_lat, q_rot, pool, out)), o._stream()), "latent_attention")
+        c_int(dt), o._stream()), "latent_attention")
     return out
 
 
