@@ -45,6 +45,9 @@
 #define TG_EPI_PLAIN 0
 #define TG_EPI_SWIGLU 1
 #define TG_EPI_RESIDUAL 2
+#define TG_EPI_GLU_CLAMP 3  // paired like SwiGLU: min(g, limit) * sigmoid(alpha * min(g, limit)) * (clamp(u, +-limit) + bias)
+#define TG_EPI_RELU_SQ 4    // relu(product)^2
+#define TG_PAIRED(E) ((E) == TG_EPI_SWIGLU || (E) == TG_EPI_GLU_CLAMP)
 
 typedef __attribute__((address_space(3))) void* tg_lds_ptr_t;
 
@@ -60,7 +63,7 @@ __global__ __launch_bounds__(512, 2) void tile_gemm_kernel(
     const uint16_t* __restrict__ a, long lda, const int* __restrict__ arow_idx,
     const uint16_t* __restrict__ w, long w_group_stride, const int* __restrict__ offsets, int n_groups, int max_rows,
     uint16_t* __restrict__ c, long ldc, const uint16_t* __restrict__ resid, long ldr,
-    int n_total, int k_total, int n_tiles) {
+    int n_total, int k_total, int n_tiles, float act_limit, float act_alpha, float act_bias) {
   extern __shared__ __attribute__((aligned(1024))) char lds[];
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -130,7 +133,7 @@ __global__ __launch_bounds__(512, 2) void tile_gemm_kernel(
         const int cb = r >> 5, ti = (r >> 4) & 1, i = r & 15;
         const int nloc = 8 * (i >> 2) + 4 * ti + (i & 3);
         int wrow;
-        if (EPI == TG_EPI_SWIGLU) {
+        if (TG_PAIRED(EPI)) {
           int col = n_idx * 128 + cb * 32 + nloc;
           if (col >= inter) col = inter - 1;
           wrow = h == 0 ? col : inter + col;
@@ -292,15 +295,21 @@ __global__ __launch_bounds__(512, 2) void tile_gemm_kernel(
 #pragma unroll
     for (int mi = 0; mi < 4; ++mi) {
       const int row = row0 + 128 * wr + 64 * mh + 16 * mi + fr;
-      if (EPI == TG_EPI_SWIGLU) {
+      if (TG_PAIRED(EPI)) {
         const int col = n_idx * 128 + wc * 32 + 8 * fq;
         float v[8];
 #pragma unroll
         for (int ni = 0; ni < 2; ++ni)
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
-            const float gt = acc[mh][0][mi][ni][e], up = acc[mh][1][mi][ni][e];
-            v[4 * ni + e] = gt / (1.f + __expf(-gt)) * up;
+            float gt = acc[mh][0][mi][ni][e], up = acc[mh][1][mi][ni][e];
+            if (EPI == TG_EPI_GLU_CLAMP) {
+              gt = fminf(gt, act_limit);
+              up = fminf(fmaxf(up, -act_limit), act_limit) + act_bias;
+              v[4 * ni + e] = gt / (1.f + __expf(-act_alpha * gt)) * up;
+            } else {
+              v[4 * ni + e] = gt / (1.f + __expf(-gt)) * up;
+            }
           }
         if (row < row_end && col < inter) {
           u32x4 o = {pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]), pack_bf16x2(v[4], v[5]), pack_bf16x2(v[6], v[7])};
@@ -316,6 +325,13 @@ __global__ __launch_bounds__(512, 2) void tile_gemm_kernel(
             for (int ni = 0; ni < 2; ++ni)
 #pragma unroll
               for (int e = 0; e < 4; ++e) v[4 * ni + e] = acc[mh][nh][mi][ni][e];
+            if (EPI == TG_EPI_RELU_SQ) {
+#pragma unroll
+              for (int p = 0; p < 8; ++p) {
+                const float r = fmaxf(v[p], 0.f);
+                v[p] = r * r;
+              }
+            }
             if (EPI == TG_EPI_RESIDUAL) {
               const u32x4 rr = *reinterpret_cast<const u32x4*>(resid + (long)row * ldr + col);
 #pragma unroll
@@ -344,19 +360,20 @@ VPSA_EXPORT int vpsa_tile_gemm_debug(int v) {
 // output row r reads A row r); w [G, N, K] contiguous; offsets [G + 1] int32 on the device with
 // offsets[G] <= max_rows, or null (one group of max_rows rows); c [max_rows, N] (SwiGLU: N / 2
 // columns), row stride ldc; epi: 0 store, 1 SwiGLU, 2 store of product + resid (row stride ldr; may
-// alias c).  Every byte offset into a and into one group of w must fit 32 bits.
+// alias c), 3 clamped gated unit (paired like SwiGLU, constants act_*), 4 squared ReLU.  Every byte offset into a and into one group of w must fit 32 bits.
 // Returns 0, or a negative number when the shape is outside what the kernel tiles.
 VPSA_EXPORT int vpsa_tile_gemm(const void* a, long lda, const void* arow_idx, const void* w, const void* offsets,
                                int n_groups, void* c, long ldc, int max_rows, int n, int k, int epi, const void* resid,
-                               long ldr, long a_rows, hipStream_t stream) {
+                               long ldr, long a_rows, float act_limit, float act_alpha, float act_bias,
+                               hipStream_t stream) {
   if (k % TG_BK != 0 || k <= 0 || n <= 0 || max_rows <= 0 || n_groups <= 0 || lda % 8 != 0 || ldc % 8 != 0) return -1;
   if (!offsets && n_groups != 1) return -1;
-  if (epi == TG_EPI_SWIGLU && (n % 2 != 0 || (n / 2) % 32 != 0)) return -1;
-  if (epi != TG_EPI_SWIGLU && n % 8 != 0) return -1;
+  if (TG_PAIRED(epi) && (n % 2 != 0 || (n / 2) % 32 != 0)) return -1;
+  if (!TG_PAIRED(epi) && n % 8 != 0) return -1;
   if (epi == TG_EPI_RESIDUAL && (!resid || ldr % 8 != 0)) return -1;
-  if (epi < 0 || epi > 2) return -1;
+  if (epi < 0 || epi > 4) return -1;
   if ((double)a_rows * (double)lda * 2.0 >= 4294967296.0 || (double)n * (double)k * 2.0 >= 4294967296.0) return -1;
-  const int n_tiles = epi == TG_EPI_SWIGLU ? (n / 2 + 127) / 128 : (n + TG_BN - 1) / TG_BN;
+  const int n_tiles = TG_PAIRED(epi) ? (n / 2 + 127) / 128 : (n + TG_BN - 1) / TG_BN;
   const int m_tiles_max = offsets ? max_rows / TG_BM + n_groups : (max_rows + TG_BM - 1) / TG_BM;
   const long blocks = (long)n_tiles * m_tiles_max;
   if (blocks > 0x7fffffffL) return -1;
@@ -372,10 +389,12 @@ VPSA_EXPORT int vpsa_tile_gemm(const void* a, long lda, const void* arow_idx, co
     }                                                                                                                \
     tile_gemm_kernel<E, D><<<dim3((unsigned)blocks), dim3(512), TG_LDS, stream>>>(                                       \
         (const uint16_t*)a, lda, (const int*)arow_idx, (const uint16_t*)w, wstride, (const int*)offsets, n_groups,   \
-        max_rows, (uint16_t*)c, ldc, (const uint16_t*)resid, ldr, n, k, n_tiles);                                    \
+        max_rows, (uint16_t*)c, ldc, (const uint16_t*)resid, ldr, n, k, n_tiles, act_limit, act_alpha, act_bias);    \
   } while (0)
   if (epi == TG_EPI_SWIGLU) TG_LAUNCH(TG_EPI_SWIGLU, 0);
   else if (epi == TG_EPI_RESIDUAL) TG_LAUNCH(TG_EPI_RESIDUAL, 0);
+  else if (epi == TG_EPI_GLU_CLAMP) TG_LAUNCH(TG_EPI_GLU_CLAMP, 0);
+  else if (epi == TG_EPI_RELU_SQ) TG_LAUNCH(TG_EPI_RELU_SQ, 0);
   else if (g_tg_debug == 1) TG_LAUNCH(TG_EPI_PLAIN, 1);
   else if (g_tg_debug == 2) TG_LAUNCH(TG_EPI_PLAIN, 2);
   else if (g_tg_debug == 3) TG_LAUNCH(TG_EPI_PLAIN, 3);

@@ -126,6 +126,53 @@ def test_attention_edges_matrix_cores(rank, rot, heads, mode, splits):
     attention_edges(torch.device("cuda"), torch.bfloat16, 3e-2, rank=rank, rot=rot, heads=heads, mode=mode, splits=splits)
 
 
+def test_gemm_epilogues():
+    """The grouped / dense prefill GEMM with the clamped gated unit and the squared ReLU in its epilogue."""
+    g = torch.Generator().manual_seed(7)
+    rows, k, inter, groups = 300, 128, 96, 3
+    x = torch.randn(rows, k, generator=g).to(torch.bfloat16)
+    w = (torch.randn(groups, 2 * inter, k, generator=g) * k ** -0.5).to(torch.bfloat16)
+    offsets = torch.tensor([0, 170, 170, 290], dtype=torch.int32)  # an empty group, rows past the last group
+    idx = torch.randperm(rows, generator=g).int()
+    got = ops.tile_gemm(x.cuda(), w.cuda(), offsets.cuda(), rows=rows, arow_idx=idx.cuda(), glu_clamp=(0.9, 1.702, 1.0))
+    for gi in range(groups):
+        lo, hi = int(offsets[gi]), int(offsets[gi + 1])
+        if hi == lo:
+            continue
+        y = x[idx[lo:hi].long()].double() @ w[gi].double().T
+        gate, up = y[:, :inter].clamp(max=0.9), y[:, inter:].clamp(-0.9, 0.9)
+        assert close(got[lo:hi], gate * torch.sigmoid(1.702 * gate) * (up + 1), 2e-2)
+    got = ops.tile_gemm(x.cuda(), w[0].cuda(), relu_sq=True)
+    assert close(got, torch.relu(x.double() @ w[0].double().T) ** 2, 2e-2)
+    assert close(ops.up_relu_sq(x.cuda(), w[0].cuda()), torch.relu(x.double() @ w[0].double().T) ** 2, 2e-2)
+
+
+def test_decode_graphs_match_eager(model_c):
+    """Decode steps replayed from captured HIP graphs (several replays per bucket, prefill steps and host
+    work between them) generate what eager steps generate."""
+    import tempfile
+
+    from vllm_production_stack_amd.engine.config import EngineConfig
+    from vllm_production_stack_amd.engine.llm_engine import LLMEngine
+    from vllm_production_stack_amd.engine.request import SamplingParams
+
+    cfg, w = model_c
+    folder = zo.save_checkpoint(cfg, w, tempfile.mkdtemp(prefix="zx-"))
+    prompts = [zc.tokens(cfg, n, 60 + n) for n in (70, 5, 130, 9, 33)]
+    outs = {}
+    for eager in (True, False):
+        ec = EngineConfig(model=folder, dtype="bfloat16", device="cuda", max_model_len=1024, max_num_seqs=8,
+                          max_num_batched_tokens=64, num_gpu_blocks_override=32, enable_prefix_caching=False,
+                          enforce_eager=eager, capture_graphs_at_start=not eager)
+        eng = LLMEngine(ec)
+        assert eng.runner.use_graphs == (not eager)
+        outs[eager] = eng.generate(prompts, SamplingParams(max_tokens=40, temperature=0.0, ignore_eos=True))
+        if not eager:
+            assert eng.runner.step_kinds["decode_graph"] > 20
+        eng.shutdown()
+    assert outs[True] == outs[False]
+
+
 @pytest.fixture(scope="module")
 def model_c():
     cfg = zo.config_c()

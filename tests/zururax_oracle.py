@@ -184,10 +184,11 @@ def config_b():
 
 
 def config_c():
-    """Cache entries of 64 + 32 and 128 + 32 values, 3 and 5 heads, a layer that reads its neighbour's entries."""
+    """Cache entries of 64 + 32 and 128 + 32 values, 3 and 5 heads, a layer that reads its neighbour's entries,
+    a mixture whose units the grouped matrix-core GEMM tiles (width and unit width multiples of 64)."""
     return make_config(83, 64, [
         layer(mixer(3, 16, 32, 8, 64, 24, base=300.0), {"kind": "dense", "ff": 72}),
-        layer(mixer(5, 8, 32, 16, 64, 32, base=300.0, kv_from=0), moe(16, 4, 2, 2, 1, shared_ff=24, scale=1.2)),
+        layer(mixer(5, 8, 32, 16, 64, 32, base=300.0, kv_from=0), moe(64, 4, 2, 2, 1, shared_ff=24, scale=1.2)),
         layer(mixer(2, 24, 32, 32, 128, 40, base=9000.0), None),
     ], embedding_scale=1.5)
 

@@ -44,7 +44,14 @@ class ZururaxLayer:
 
 
 class ZururaxModel:
-    graph_capturable = False  # the expert loop reads the per-expert row counts on the host
+    @property
+    def graph_capturable(self) -> bool:
+        """Decode steps can be captured when no layer's mixture falls back to the per-unit loop, which
+        reads the row counts on the host (shapes the grouped GEMM does not tile, fp32)."""
+        return self.dtype == torch.bfloat16 and self.device.type == "cuda" and all(
+            lw.w13 is None or ops.moe_glu_grouped_supported(torch.empty((1, self.cfg.hidden_size), dtype=self.dtype,
+                                                                         device=self.device), lw.w13, lw.w2)
+            for lw in self.layers)
 
     def __init__(self, cfg: ModelConfig, dtype: torch.dtype, device: torch.device, max_model_len: int):
         if get_tp().size != 1 or get_pp().size != 1:
@@ -168,10 +175,10 @@ class ZururaxModel:
         m: LatentMixerSpec = lw.spec.mixer
         eps = self.cfg.norm_eps
         t = h.shape[0]
-        proj = F.linear(h, lw.w_in)
+        proj = ops.linear(h, lw.w_in)
         col = m.q_rank
         cq = ops.rms_norm_rows(proj[:, :col], lw.dq_norm, eps)
-        q = F.linear(cq, lw.w_uq).view(t, m.heads, m.dim + m.rot_dim)
+        q = ops.linear(cq, lw.w_uq).view(t, m.heads, m.dim + m.rot_dim)
         ops.rope_pairs(q, meta.positions, lw.cos_sin, m.dim, m.rope_dims)
         if m.kv_from is None:
             ops.latent_kv_write(proj[:, col:col + m.entry], lw.dkv_norm, meta.positions, meta.slots, lw.cos_sin, pool,
@@ -194,7 +201,7 @@ class ZururaxModel:
         o = torch.bmm(o_lat.transpose(0, 1), lw.w_uv.transpose(1, 2)).transpose(0, 1).contiguous()
         if m.out_gate:
             ops.sigmoid_gate(o, proj[:, col:col + m.heads])
-        return F.linear(o.view(t, m.heads * m.vdim), lw.w_o)
+        return ops.linear(o.view(t, m.heads * m.vdim), lw.w_o)
 
     def _moe(self, lw: ZururaxLayer, h: torch.Tensor, residual: torch.Tensor) -> None:
         """Adds the mixture's output for rows h into the fp32 residual stream."""
@@ -204,7 +211,12 @@ class ZururaxModel:
         w, ids, gate = ops.group_topk(logits, f.experts, f.groups, f.keep, f.top, f.route_scale, extra=f.shared_ff > 0)
         shared = None
         if f.shared_ff:
-            shared = F.linear(ops.glu_clamp(F.linear(h, lw.w_sh13), f.shared_limit, GLU_ALPHA, GLU_UP_BIAS), lw.w_sh2)
+            shared = ops.linear(ops.gate_up_glu_clamp(h, lw.w_sh13, f.shared_limit, GLU_ALPHA, GLU_UP_BIAS), lw.w_sh2)
+        if ops.moe_glu_grouped_supported(h, lw.w13, lw.w2):
+            ys, pos = ops.moe_glu_grouped(h, lw.w13, lw.w2, ids, f.limit, GLU_ALPHA, GLU_UP_BIAS)
+            ops.moe_finish(residual, ys, w, pos, shared, gate)
+            return
+        # the CPU, fp32, and shapes the grouped kernel does not tile: unit by unit on the sorted rows
         offsets, pos, sorted_tok = ops.moe_align(ids, f.experts)
         xs = ops.gather_rows(h, sorted_tok)
         ys = torch.empty((t * f.top, h.shape[1]), dtype=h.dtype, device=h.device)
@@ -230,7 +242,7 @@ class ZururaxModel:
                 h = ops.add_rms_norm(x, d, lw.norm2, eps, self.dtype)
                 d = None
                 if f.kind == "dense":
-                    d = F.linear(ops.relu_sq(F.linear(h, lw.w_up)), lw.w_down)
+                    d = ops.linear(ops.up_relu_sq(h, lw.w_up), lw.w_down)
                 else:
                     self._moe(lw, h, x)
             if self.layer_probe is not None:
@@ -241,4 +253,4 @@ class ZururaxModel:
         return ops.add_rms_norm(x, d, self.norm, eps, self.dtype)
 
     def compute_logits(self, hidden: torch.Tensor) -> torch.Tensor:
-        return F.linear(hidden, self.lm_head)
+        return ops.linear(hidden, self.lm_head)

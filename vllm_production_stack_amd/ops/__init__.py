@@ -1186,22 +1186,26 @@ def tile_gemm_supported(n: int, k: int, silu_mul: bool = False) -> bool:
     return k % 64 == 0 and n % 8 == 0 and (not silu_mul or (n // 2) % 32 == 0) and n * k * 2 < 2 ** 32
 
 
-def tile_gemm(a, w, offsets=None, rows=None, arow_idx=None, silu_mul=False, residual=None, out=None):
+def tile_gemm(a, w, offsets=None, rows=None, arow_idx=None, silu_mul=False, residual=None, out=None, glu_clamp=None,
+              relu_sq=False):
     """The prefill GEMM (``csrc/kernels/tile_gemm.hip``): out[r] = epilogue(a[arow_idx[r] or r] @ w[g]^T).
 
     a [*, K] bf16; w [N, K] (dense) or [G, N, K] (grouped, with offsets [G + 1] int32 ON THE DEVICE:
     group g owns output rows offsets[g] .. offsets[g+1], no host synchronisation).  silu_mul: w is
     [gate rows | up rows], out = silu(gate) * up, [rows, N / 2].  residual [rows, N]: out = product +
-    residual (``out`` may be ``residual`` itself).  Rows at or past offsets[G] are left unwritten."""
+    residual (``out`` may be ``residual`` itself).  glu_clamp = (limit, alpha, bias): w is [gate rows | up
+    rows] as for silu_mul, out = min(g, limit) * sigmoid(alpha min(g, limit)) * (clamp(u, +-limit) + bias).
+    relu_sq: out = relu(product)^2.  Rows at or past offsets[G] are left unwritten."""
+    paired = silu_mul or glu_clamp is not None
     if w.dim() == 2:
         w = w.unsqueeze(0)
     g, n, k = w.shape
     if rows is None:
         rows = a.shape[0] if arow_idx is None else arow_idx.numel()
-    n_out = n // 2 if silu_mul else n
+    n_out = n // 2 if paired else n
     _bf16_cuda(a, w, residual)
     assert w.is_contiguous() and a.stride(-1) == 1 and a.shape[1] == k
-    assert not (silu_mul and residual is not None)
+    assert sum((silu_mul, glu_clamp is not None, relu_sq, residual is not None)) <= 1
     if offsets is not None:
         assert offsets.dtype == torch.int32 and offsets.numel() == g + 1 and offsets.is_cuda
     else:
@@ -1213,11 +1217,12 @@ def tile_gemm(a, w, offsets=None, rows=None, arow_idx=None, silu_mul=False, resi
     assert out.stride(-1) == 1 and out.shape[0] >= rows and out.shape[1] == n_out
     if residual is not None:
         assert residual.stride(-1) == 1 and residual.shape[0] >= rows and residual.shape[1] == n_out
-    epi = 1 if silu_mul else (2 if residual is not None else 0)
+    epi = 1 if silu_mul else 2 if residual is not None else 3 if glu_clamp is not None else 4 if relu_sq else 0
+    lim, alpha, bias = glu_clamp if glu_clamp is not None else (0.0, 1.0, 0.0)
     rc = _kernels().vpsa_tile_gemm(_p(a), c_long(a.stride(0)), _p(arow_idx), _p(w), _p(offsets), c_int(g), _p(out),
                                    c_long(out.stride(0)), c_int(rows), c_int(n), c_int(k), c_int(epi), _p(residual),
                                    c_long(residual.stride(0) if residual is not None else 0), c_long(a.shape[0]),
-                                   _stream())
+                                   c_float(lim), c_float(alpha), c_float(bias), _stream())
     _check(rc, "tile_gemm")
     return out
 
@@ -1316,5 +1321,6 @@ def lora_expand(h, bs, slots, y, r_pad):
 
 
 # --------------------------------------------------------------------------- latent attention, group routing, fp32 residual
-from .latent import (add_rms_norm, build_latent_tiles, embed_scale, gather_rows, glu_clamp, group_topk, latent_attention,  # noqa: E402,F401
+from .latent import (add_rms_norm, build_latent_tiles, embed_scale, gate_up_glu_clamp, gather_rows, glu_clamp,  # noqa: E402,F401
+                     group_topk, latent_attention, moe_glu_grouped, moe_glu_grouped_supported, up_relu_sq,
                      latent_kv_write, latent_mfma_supported, moe_finish, relu_sq, rms_norm_rows, rope_pairs, sigmoid_gate)

@@ -301,3 +301,40 @@ def moe_finish(residual, y, weights, pos, shared=None, gate=None):
                                           o._p(shared), o._p(gate), c_int(t), c_int(n), c_int(_dt(y, shared)),
                                           o._stream()), "moe_finish")
     return residual
+
+
+def gate_up_glu_clamp(x, w_gate_up, limit: float, alpha: float = 1.702, up_bias: float = 1.0):
+    """The clamped gated unit's activation of ``x @ [Wg; Wu].T``: in the epilogue of the prefill GEMM when
+    that kernel takes the shape, else the projection (``ops.linear``) and the activation kernel."""
+    o = _ops()
+    rows = o.tile_rows(x, w_gate_up, True) if x.is_cuda else 0
+    if rows:
+        return o.tile_gemm(x, w_gate_up, glu_clamp=(limit, alpha, up_bias))
+    return glu_clamp(o.linear(x, w_gate_up), limit, alpha, up_bias)
+
+
+def up_relu_sq(x, w_up):
+    """relu(x @ W.T)^2, fused into the prefill GEMM's epilogue when that kernel takes the shape."""
+    o = _ops()
+    rows = o.tile_rows(x, w_up) if x.is_cuda else 0
+    if rows:
+        return o.tile_gemm(x, w_up, relu_sq=True)
+    return relu_sq(o.linear(x, w_up))
+
+
+def moe_glu_grouped_supported(x, w13, w2) -> bool:
+    o = _ops()
+    return (x.is_cuda and x.dtype == torch.bfloat16 and x.is_contiguous() and w13.is_contiguous() and w2.is_contiguous()
+            and o.tile_gemm_supported(w13.shape[1], w13.shape[2], True) and o.tile_gemm_supported(w2.shape[1], w2.shape[2]))
+
+
+def moe_glu_grouped(x, w13, w2, ids, limit: float, alpha: float = 1.702, up_bias: float = 1.0):
+    """Clamped gated units of a mixture over the device-sorted (token, unit) pairs: two grouped
+    matrix-core GEMMs (the first gathers its token rows and applies the activation in its epilogue).
+    The host never reads the per-unit counts: no synchronisation, HIP-graph capturable.
+    Returns (y [T * K, hidden] in sorted order, pos [T * K]: the sorted row of pair t * K + k)."""
+    o = _ops()
+    t, k = ids.shape
+    offsets, pos, sorted_tok = o.moe_align(ids, w13.shape[0])
+    act = o.tile_gemm(x, w13, offsets, rows=t * k, arow_idx=sorted_tok, glu_clamp=(limit, alpha, up_bias))
+    return o.tile_gemm(act, w2, offsets, rows=t * k), pos
