@@ -110,6 +110,15 @@ def parse() -> argparse.Namespace:
                          "+ 6 decode replicas behind the router in disaggregated_prefill mode; 'multimodel' = six "
                          "replicas of --model + a TP2 Mixtral-8x7B replica, kvaware routing, shared KV cache server. "
                          "VPSA_BENCH_SINGLE_DEVICE=1 (+ --num-gpu-blocks) rehearses either on one card")
+    ap.add_argument("--arch-compare", default="",
+                    help="instead of the serving benchmark: prefill and decode throughput of this decoder design "
+                         "('zururax') beside the closest existing design at equal size (benchmarks/arch_compare.py)")
+    ap.add_argument("--arch-sizes", default="s,m")
+    ap.add_argument("--arch-prompt", type=int, default=4096, help="--arch-compare: prompt length")
+    ap.add_argument("--arch-prompts", type=int, default=4, help="--arch-compare: prompts per prefill measurement")
+    ap.add_argument("--arch-batch", type=int, default=32, help="--arch-compare: decode batch")
+    ap.add_argument("--arch-context", type=int, default=2048, help="--arch-compare: context per decoding sequence")
+    ap.add_argument("--arch-decode-steps", type=int, default=48)
     ap.add_argument("--device", default="cuda", help="cpu runs a plumbing rehearsal (tiny models)")
     # internal: load-generator mode
     ap.add_argument("--client", action="store_true")
@@ -597,6 +606,12 @@ def main() -> None:
     a = parse()
     if a.client:
         client_main(a)
+        return
+    if a.arch_compare:
+        sys.path.insert(0, os.path.join(ROOT, "benchmarks"))
+        import arch_compare
+
+        arch_compare.main(a)
         return
     if a.layout:
         sys.path.insert(0, os.path.join(ROOT, "benchmarks"))

@@ -15,7 +15,8 @@
 // loads), stores its rows into the K image and the 4 x 8 transpose into the V^T image.  The keys of
 // the V^T image are permuted so that the 8 keys a lane owns in the S^T accumulators (v_mfma 16x16x32:
 // lane = query l % 16, keys 4 (l / 16) + e of four 16-key tiles) are 16 contiguous bytes: P goes from
-// the S accumulators into the second product without leaving the lane.
+// the S accumulators into the second product without leaving the lane.  (The 16-byte chunks of a V^T row
+// are XOR-swizzled with (row / 8) % 8: the transposing stores of neighbouring lanes lie 8 rows apart.)
 // The next page's global loads are issued before the current page is multiplied.
 //
 // Softmax state (running max, sum) is fp32 per slot; an optional per-head sink logit starts the state
@@ -116,15 +117,18 @@ __global__ __launch_bounds__(256) void latent_mfma_kernel(
 #pragma unroll
       for (int i = 0; i < 4; ++i) *reinterpret_cast<u32x4*>(kimg + (4 * kq + i) * PK + 16 * dc) = rb[b][i];
       // keys 4 kq .. 4 kq + 3 = 16 n + 4 gg + e  ->  image position (n / 2) * 32 + gg * 8 + (n % 2) * 4 + e
+      // = 16-byte chunk (n / 2) * 4 + gg, half n % 2.  Rows 8 dc .. 8 dc + 7 are written by one lane and
+      // consecutive lanes hold consecutive dc, 8 rows = 1152 B apart: the chunk index is XORed with dc % 8
+      // (= (row / 8) % 8, which the reader undoes) so that those lanes spread over the banks.
       const int n = kq >> 2, gg = kq & 3;
-      const int kpos = (n >> 1) * 32 + gg * 8 + (n & 1) * 4;
+      const int koff = ((((n >> 1) * 4 + gg) ^ (dc & 7)) << 4) + ((n & 1) << 3);
 #pragma unroll
       for (int w = 0; w < 4; ++w) {
         const uint32_t a0 = rb[b][0][w], a1 = rb[b][1][w], a2 = rb[b][2][w], a3 = rb[b][3][w];
         u32x2 even = {(a0 & 0xffffu) | (a1 << 16), (a2 & 0xffffu) | (a3 << 16)};
         u32x2 odd = {(a0 >> 16) | (a1 & 0xffff0000u), (a2 >> 16) | (a3 & 0xffff0000u)};
-        *reinterpret_cast<u32x2*>(vimg + (8 * dc + 2 * w) * PV + 2 * kpos) = even;
-        *reinterpret_cast<u32x2*>(vimg + (8 * dc + 2 * w + 1) * PV + 2 * kpos) = odd;
+        *reinterpret_cast<u32x2*>(vimg + (8 * dc + 2 * w) * PV + koff) = even;
+        *reinterpret_cast<u32x2*>(vimg + (8 * dc + 2 * w + 1) * PV + koff) = odd;
       }
     }
 #pragma unroll
@@ -191,7 +195,8 @@ __global__ __launch_bounds__(256) void latent_mfma_kernel(
       o[dt] *= corr;
 #pragma unroll
       for (int kk = 0; kk < 2; ++kk) {
-        const bf16x8 a = *reinterpret_cast<const bf16x8*>(vimg + (16 * dt + c16) * PV + (kk * 32 + g * 8) * 2);
+        const int vrow = 16 * dt + c16;
+        const bf16x8 a = *reinterpret_cast<const bf16x8*>(vimg + vrow * PV + (((kk * 4 + g) ^ ((vrow >> 3) & 7)) << 4));
         o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pf[kk], o[dt], 0, 0, 0);
       }
     }
