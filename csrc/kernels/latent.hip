@@ -230,7 +230,7 @@ __global__ __launch_bounds__(256) void latent_attention_kernel(
         acc[c] = a;
       }
     }
-    __syncthreads();  // ps is rewritten by the next round
+    __syncthreads();  // ps is rewritten by the next 256 keys
   }
   const float inv = l > 0.f ? 1.f / l : 0.f;
 #pragma unroll

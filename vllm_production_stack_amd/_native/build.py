@@ -50,6 +50,12 @@ TARGETS = {
 SOURCE_FLAGS = {
     "kernels/attention.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
 }
+# sources that keep the compiler's default for packed fp32.  attention.hip: built with the feature
+# switched off, the GQA prefill path gives different logits in the mixed-adapter engine test
+# (tests/test_engine_gpu.py::test_adapters_on_the_gpu_match_merged_weights_in_a_mixed_batch: cosine 0.989
+# where 0.995 is required; every other object was exchanged one by one and does not matter).  Its kernels
+# allocate most of the register file by hand, so it stays as it was measured until that is understood.
+NO_HIP_FLAGS = {"kernels/attention.hip"}
 
 # standalone executables: name -> (kind, sources, flags)
 BINARIES = {
@@ -99,7 +105,7 @@ def build_target(name: str, force: bool = False) -> Path | None:
             obj = objdir / (path.stem + ".o")
             if force or _stale(obj, [path]):
                 _run([HIPCC, "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden",
-                      *HIP_FLAGS, "-I", str(CSRC), *SOURCE_FLAGS.get(src, []), "-c", str(path), "-o", str(obj)])
+                      *([] if src in NO_HIP_FLAGS else HIP_FLAGS), "-I", str(CSRC), *SOURCE_FLAGS.get(src, []), "-c", str(path), "-o", str(obj)])
             objs.append(str(obj))
         cmd = [HIPCC, "--offload-arch=gfx950", *shared, *objs, "-o", str(out), *flags]
     elif kind == "hip":
