@@ -65,6 +65,7 @@ __global__ __launch_bounds__(256) void latent_mfma_kernel(
   if (t.seq < 0) return;
   const int slot = wave * 16 + c16;
   const bool valid = slot < t.n_tok * t.hcount;
+  const bool wave_active = wave * 16 < t.n_tok * t.hcount;  // wave-uniform
   const int tok = valid ? slot / t.hcount : 0;
   const int head = t.head0 + (valid ? slot % t.hcount : 0);
   const long row = t.row0 + tok;
@@ -144,6 +145,7 @@ __global__ __launch_bounds__(256) void latent_mfma_kernel(
     stash();
     __syncthreads();
     if (p + 1 < p_end) fetch(p + 1);  // in flight while this page is multiplied
+    if (!wave_active) continue;       // a wave without slots (decode rows of few heads) only helps staging
 
     f32x4 s[4];
 #pragma unroll
