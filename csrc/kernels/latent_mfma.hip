@@ -139,6 +139,14 @@ __global__ __launch_bounds__(256) void latent_mfma_kernel(
     }
   };
 
+  // V^T fragment of (d tile dt, key half kk): row 16 dt + c16, chunk (4 kk + g) ^ ((row / 8) % 8); the row's
+  // share of the swizzle is (2 dt) % 8 | c16 / 8, so eight lane offsets cover every dt
+  int voff[2][4];
+#pragma unroll
+  for (int kk = 0; kk < 2; ++kk)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) voff[kk][j] = c16 * PV + (((kk * 4 + g) ^ (c16 >> 3) ^ (2 * j)) << 4);
+
   if (p_begin < p_end) fetch(p_begin);
   for (int p = p_begin; p < p_end; ++p) {
     __syncthreads();  // the previous page's fragment reads are done
@@ -192,16 +200,12 @@ __global__ __launch_bounds__(256) void latent_mfma_kernel(
                  pack_bf16x2(s[2 * kk + 1][0], s[2 * kk + 1][1]), pack_bf16x2(s[2 * kk + 1][2], s[2 * kk + 1][3])};
       pf[kk] = __builtin_bit_cast(bf16x8, w);
     }
-    if (!__all(corr == 1.f)) {  // the running maxima settle after a few pages: most pages rescale nothing
-#pragma unroll
-      for (int dt = 0; dt < DT; ++dt) o[dt] *= corr;
-    }
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) {
+      o[dt] *= corr;
 #pragma unroll
       for (int kk = 0; kk < 2; ++kk) {
-        const int vrow = 16 * dt + c16;
-        const bf16x8 a = *reinterpret_cast<const bf16x8*>(vimg + vrow * PV + (((kk * 4 + g) ^ ((vrow >> 3) & 7)) << 4));
+        const bf16x8 a = *reinterpret_cast<const bf16x8*>(vimg + voff[kk][dt & 3] + dt * 16 * PV);
         o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pf[kk], o[dt], 0, 0, 0);
       }
     }
