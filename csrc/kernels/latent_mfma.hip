@@ -200,9 +200,12 @@ __global__ __launch_bounds__(256) void latent_mfma_kernel(
                  pack_bf16x2(s[2 * kk + 1][0], s[2 * kk + 1][1]), pack_bf16x2(s[2 * kk + 1][2], s[2 * kk + 1][3])};
       pf[kk] = __builtin_bit_cast(bf16x8, w);
     }
+    if (!__all(corr == 1.f)) {
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) o[dt] *= corr;
+    }
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) {
-      o[dt] *= corr;
 #pragma unroll
       for (int kk = 0; kk < 2; ++kk) {
         const bf16x8 a = *reinterpret_cast<const bf16x8*>(vimg + voff[kk][dt & 3] + dt * 16 * PV);
