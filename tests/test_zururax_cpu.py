@@ -203,3 +203,36 @@ def test_batches_and_reuse(model_a):
 def test_greedy_generation(model_a, model_b):
     zc.check_generate(DEV, DT, *model_a)
     zc.check_generate(DEV, DT, *model_b, n_new=30)
+
+
+def test_replay_command(tmp_path):
+    """bin/trace_run: the line protocol, the logits files, requests that end and whose pages are used again."""
+    import json
+    import os
+    import subprocess
+    import sys
+
+    import numpy as np
+
+    cfg = zo.config_b()
+    w = zo.make_weights(cfg, seed=9)
+    folder = zo.save_checkpoint(cfg, w, tmp_path / "m")
+    a, b = zc.tokens(cfg, 100, 1), zc.tokens(cfg, 70, 2)
+    steps = [
+        {"step": 0, "entries": [{"id": "a", "tokens": a[:64], "want": [0, 63]}], "end": []},
+        {"step": 1, "entries": [{"id": "a", "tokens": a[64:99], "want": []}, {"id": "b", "tokens": b[:3], "want": [2]}], "end": []},
+        {"step": 2, "entries": [{"id": "b", "tokens": b[3:], "want": [66]}, {"id": "a", "tokens": a[99:], "want": [0]}], "end": ["a", "b"]},
+        {"step": 3, "entries": [{"id": "c", "tokens": a, "want": [99]}], "end": ["c"]},  # its pages were a's or b's
+    ]
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    out = tmp_path / "out"
+    p = subprocess.run([sys.executable, os.path.join(root, "bin", "trace_run"), "--model", folder, "--dtype", "float32",
+                        "--out", str(out), "--max-tokens", "256", "--device", "cpu"],
+                       input="".join(json.dumps(s) + "\n" for s in steps), capture_output=True, text=True, timeout=300)
+    assert p.returncode == 0, p.stderr[-2000:]
+    assert [ln for ln in p.stdout.splitlines() if ln.startswith("done")] == ["done 0", "done 1", "done 2", "done 3"]
+    la, lb = zo.forward(cfg, w, a), zo.forward(cfg, w, b)
+    want = {0: la[[0, 63]], 1: lb[[2]], 2: torch.stack([lb[69], la[99]]), 3: la[[99]]}
+    for n, ref in want.items():
+        got = torch.from_numpy(np.fromfile(out / f"{n}.f32", dtype="<f4").reshape(-1, cfg["vocab"]))
+        assert got.shape == ref.shape and zo.rel_error(got, ref) < TOL

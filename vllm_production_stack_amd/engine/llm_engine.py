@@ -86,6 +86,10 @@ class LLMEngine:
             # the tiers move whole pages of one process's pool
             log.warning("KV offload / transfer tiers are disabled for tensor/pipeline-parallel replicas")
             return
+        if self.runner.custom_pages:
+            # the tiers' codecs and page movers know the [layer][K|V][head] page of the GQA decoders
+            log.warning("KV offload / transfer tiers are disabled for models that lay out their cache pages themselves")
+            return
         from ..kv.connector import KVConnector
 
         self.connector = KVConnector(self, off, kvt)
