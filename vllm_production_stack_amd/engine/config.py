@@ -113,7 +113,7 @@ def zururax_config(name: str, vocab: int, width: int, layers: list[dict], embedd
         num_heads=max(s.mixer.heads for s in specs), num_kv_heads=1,
         head_dim=max(s.mixer.dim + s.mixer.rot_dim for s in specs), norm_eps=float(norm_eps),
         max_position_embeddings=max_position_embeddings, embedding_scale=float(embedding_scale),
-        layer_specs=specs)
+        layer_specs=specs, bos_token_id=0, eos_token_id=-1)  # the design names no special tokens
 
 
 @dataclass
