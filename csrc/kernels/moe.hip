@@ -318,7 +318,7 @@ template <int TT>
 __global__ __launch_bounds__(256) void moe_mfma_gate_up_kernel(
     const uint16_t* __restrict__ x, const uint16_t* __restrict__ w13,
     const int* __restrict__ offsets, const int* __restrict__ sorted_tok,
-    uint16_t* __restrict__ act, int hidden, int inter) {
+    uint16_t* __restrict__ act, int hidden, int inter, float act_limit, float act_alpha, float act_bias) {
   const int e = blockIdx.y;
   const int r0 = offsets[e];
   const int n_e = offsets[e + 1] - r0;
@@ -368,8 +368,14 @@ __global__ __launch_bounds__(256) void moe_mfma_gate_up_kernel(
         float v[4];
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-          const float gt = accg[tt][r];
-          v[r] = gt / (1.f + __expf(-gt)) * accu[tt][r];
+          float gt = accg[tt][r], up = accu[tt][r];
+          if (act_limit > 0.f) {  // clamped gated unit: min(g, limit) * sigmoid(alpha g) * (clamp(u) + bias)
+            gt = fminf(gt, act_limit);
+            up = fminf(fmaxf(up, -act_limit), act_limit) + act_bias;
+            v[r] = gt / (1.f + __expf(-act_alpha * gt)) * up;
+          } else {
+            v[r] = gt / (1.f + __expf(-gt)) * up;
+          }
         }
         u32x2 o;
         o[0] = pack_bf16x2(v[0], v[1]);
@@ -443,10 +449,10 @@ __global__ __launch_bounds__(256) void moe_mfma_down_kernel(
 template <int TT>
 static void launch_moe_mfma(const void* x, const void* w13, const void* w2, const int* offsets,
                             const int* sorted_tok, void* act, void* y, int n_experts, int hidden,
-                            int inter, hipStream_t stream) {
+                            int inter, float act_limit, float act_alpha, float act_bias, hipStream_t stream) {
   hipLaunchKernelGGL(moe_mfma_gate_up_kernel<TT>, dim3(inter / 64, n_experts), dim3(256), 0, stream,
                      (const uint16_t*)x, (const uint16_t*)w13, offsets, sorted_tok, (uint16_t*)act,
-                     hidden, inter);
+                     hidden, inter, act_limit, act_alpha, act_bias);
   hipLaunchKernelGGL(moe_mfma_down_kernel<TT>, dim3(hidden / 16, n_experts), dim3(256), 0, stream,
                      (const uint16_t*)act, (const uint16_t*)w2, offsets, (uint16_t*)y, hidden, inter);
 }
@@ -454,20 +460,33 @@ static void launch_moe_mfma(const void* x, const void* w13, const void* w2, cons
 // x [tokens, hidden]; w13 [E, 2*inter, hidden]; w2 [E, hidden, inter]; offsets [E+1] and
 // sorted_tok [tokens*topk] from vpsa_moe_align; act [tokens*topk, inter] and
 // y [tokens*topk, hidden] are workspaces in expert-sorted row order.
-VPSA_EXPORT int vpsa_moe_mfma(const void* x, const void* w13, const void* w2, const int* offsets,
-                              const int* sorted_tok, void* act, void* y, int tokens, int topk,
-                              int n_experts, int hidden, int inter, hipStream_t stream) {
+// act_limit > 0: the clamped gated unit (limit, alpha, bias) instead of SwiGLU.
+VPSA_EXPORT int vpsa_moe_mfma_act(const void* x, const void* w13, const void* w2, const int* offsets,
+                                  const int* sorted_tok, void* act, void* y, int tokens, int topk,
+                                  int n_experts, int hidden, int inter, float act_limit, float act_alpha,
+                                  float act_bias, hipStream_t stream) {
   if (tokens * topk <= 0) return 0;
-  if (n_experts > MAX_EXPERTS) return -1;
+  if (n_experts > ALIGN_MAX_EXPERTS) return -1;
   if (hidden % (32 * MOE_KU) != 0 || hidden % 16 != 0 || inter % 64 != 0 ||
       (inter / 4) % (32 * MOE_KU) != 0)
     return -1;
   // an expert sees each token at most once: tokens bounds its row count
   if (tokens <= 16)
-    launch_moe_mfma<1>(x, w13, w2, offsets, sorted_tok, act, y, n_experts, hidden, inter, stream);
+    launch_moe_mfma<1>(x, w13, w2, offsets, sorted_tok, act, y, n_experts, hidden, inter, act_limit, act_alpha,
+                       act_bias, stream);
   else if (tokens <= 32)
-    launch_moe_mfma<2>(x, w13, w2, offsets, sorted_tok, act, y, n_experts, hidden, inter, stream);
+    launch_moe_mfma<2>(x, w13, w2, offsets, sorted_tok, act, y, n_experts, hidden, inter, act_limit, act_alpha,
+                       act_bias, stream);
   else
-    launch_moe_mfma<4>(x, w13, w2, offsets, sorted_tok, act, y, n_experts, hidden, inter, stream);
+    launch_moe_mfma<4>(x, w13, w2, offsets, sorted_tok, act, y, n_experts, hidden, inter, act_limit, act_alpha,
+                       act_bias, stream);
   return 0;
+}
+
+VPSA_EXPORT int vpsa_moe_mfma(const void* x, const void* w13, const void* w2, const int* offsets,
+                              const int* sorted_tok, void* act, void* y, int tokens, int topk,
+                              int n_experts, int hidden, int inter, hipStream_t stream) {
+  if (n_experts > MAX_EXPERTS) return -1;
+  return vpsa_moe_mfma_act(x, w13, w2, offsets, sorted_tok, act, y, tokens, topk, n_experts, hidden, inter, 0.f,
+                           1.f, 0.f, stream);
 }

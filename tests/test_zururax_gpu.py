@@ -147,6 +147,27 @@ def test_gemm_epilogues():
     assert close(ops.up_relu_sq(x.cuda(), w[0].cuda()), torch.relu(x.double() @ w[0].double().T) ** 2, 2e-2)
 
 
+@pytest.mark.parametrize("tokens", [1, 5, 40, 100])
+def test_mixture_units_small_and_large_batches(tokens):
+    """The routed units over sorted pairs: the weight-streaming kernels of decode-sized batches and the
+    grouped prefill GEMM give what the float64 definition gives."""
+    g = torch.Generator().manual_seed(tokens)
+    e, hidden, inter, top = 6, 128, 512, 2
+    x = torch.randn(tokens, hidden, generator=g).to(torch.bfloat16)
+    w13 = (torch.randn(e, 2 * inter, hidden, generator=g) * hidden ** -0.5).to(torch.bfloat16)
+    w2 = (torch.randn(e, hidden, inter, generator=g) * inter ** -0.5).to(torch.bfloat16)
+    ids = torch.stack([torch.randperm(e, generator=g)[:top] for _ in range(tokens)]).int()
+    assert ops.moe_glu_grouped_supported(x.cuda(), w13.cuda(), w2.cuda())
+    y, pos = ops.moe_glu_grouped(x.cuda(), w13.cuda(), w2.cuda(), ids.cuda(), 1.1, 1.702, 1.0)
+    for t in range(tokens):
+        for k in range(top):
+            ex = int(ids[t, k])
+            gu = x[t].double() @ w13[ex].double().T
+            gate, up = gu[:inter].clamp(max=1.1), gu[inter:].clamp(-1.1, 1.1)
+            want = (gate * torch.sigmoid(1.702 * gate) * (up + 1)) @ w2[ex].double().T
+            assert close(y[int(pos[t * top + k])], want, 3e-2), (t, k)
+
+
 def test_decode_graphs_match_eager(model_c):
     """Decode steps replayed from captured HIP graphs (several replays per bucket, prefill steps and host
     work between them) generate what eager steps generate."""

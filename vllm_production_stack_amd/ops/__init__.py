@@ -40,6 +40,7 @@ def _kernels():
             "vpsa_embed_scale", "vpsa_add_rmsnorm", "vpsa_rmsnorm_rows", "vpsa_latent_kv_write", "vpsa_rope_pairs",
             "vpsa_latent_attention", "vpsa_sigmoid_gate", "vpsa_relu_sq", "vpsa_glu_clamp", "vpsa_group_topk",
             "vpsa_gather_rows", "vpsa_moe_finish", "vpsa_latent_mfma_supported", "vpsa_latent_attention_mfma",
+            "vpsa_moe_mfma_act",
         ):
             getattr(lib, name).restype = c_int
         lib.vpsa_prefill_split_record_bytes.restype = c_long

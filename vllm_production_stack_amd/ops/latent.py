@@ -336,5 +336,16 @@ def moe_glu_grouped(x, w13, w2, ids, limit: float, alpha: float = 1.702, up_bias
     o = _ops()
     t, k = ids.shape
     offsets, pos, sorted_tok = o.moe_align(ids, w13.shape[0])
+    hidden, inter = x.shape[1], w2.shape[2]
+    if t <= o.MOE_MFMA_MAX_TOKENS and o.moe_mfma_supported(hidden, inter) and limit > 0:
+        # decode-sized batches: each routed unit's weights streamed once against its few tokens
+        # (the kernels of the top-k softmax mixtures, with this unit's activation)
+        act = torch.empty((t * k, inter), dtype=x.dtype, device=x.device)
+        y = torch.empty((t * k, hidden), dtype=x.dtype, device=x.device)
+        o._check(o._kernels().vpsa_moe_mfma_act(o._p(x), o._p(w13), o._p(w2), o._p(offsets), o._p(sorted_tok), o._p(act),
+                                                o._p(y), c_int(t), c_int(k), c_int(w13.shape[0]), c_int(hidden),
+                                                c_int(inter), c_float(limit), c_float(alpha), c_float(up_bias),
+                                                o._stream()), "moe_mfma_act")
+        return y, pos
     act = o.tile_gemm(x, w13, offsets, rows=t * k, arow_idx=sorted_tok, glu_clamp=(limit, alpha, up_bias))
     return o.tile_gemm(act, w2, offsets, rows=t * k), pos
