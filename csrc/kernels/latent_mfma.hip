@@ -300,8 +300,17 @@ int launch(const void* q_lat, long ql_row, long ql_head, const void* q_rot, long
 }  // namespace
 
 // 1 when the matrix-core kernel tiles entries of this shape
+// (latent entries: rank + rot; expanded per-head entries of a prefill: value | unrotated key | rotated key part,
+// rank = value channels, rot = the key's channels)
+#define LAT_SHAPES(X) \
+  X(64, 32) X(64, 64) X(128, 32) X(128, 64) X(256, 32) X(256, 64) X(512, 32) X(512, 64) \
+  X(32, 64) X(64, 96) X(64, 128) X(128, 128) X(128, 192)
+
 VPSA_EXPORT int vpsa_latent_mfma_supported(int rank, int rot) {
-  return ((rank == 64 || rank == 128 || rank == 256 || rank == 512) && (rot == 32 || rot == 64)) ? 1 : 0;
+#define LAT_IS(R, C) if (rank == R && rot == C) return 1;
+  LAT_SHAPES(LAT_IS)
+#undef LAT_IS
+  return 0;
 }
 
 // tiles: int32 [n_tiles, 6] = (sequence, first query row, tokens, position of the first token, first head,
@@ -321,15 +330,8 @@ VPSA_EXPORT int vpsa_latent_attention_mfma(const void* q_lat, long ql_row, long 
 #define LAT_CASE(R, C)                                                                                              \
   if (rank == R && rot == C)                                                                                        \
     return launch<R, C>(q_lat, ql_row, ql_head, q_rot, qr_row, qr_head, cache, page_stride, block_tables, bt_stride, \
-                        tiles, positions, n_tiles, heads, sink, out, o_row, o_head, scale, splits, ws_o, ws_ml, st)
-  LAT_CASE(64, 32);
-  LAT_CASE(64, 64);
-  LAT_CASE(128, 32);
-  LAT_CASE(128, 64);
-  LAT_CASE(256, 32);
-  LAT_CASE(256, 64);
-  LAT_CASE(512, 32);
-  LAT_CASE(512, 64);
+                        tiles, positions, n_tiles, heads, sink, out, o_row, o_head, scale, splits, ws_o, ws_ml, st);
+  LAT_SHAPES(LAT_CASE)
 #undef LAT_CASE
   return -1;
 }

@@ -117,7 +117,8 @@ def test_attention_edges(dtype):
     attention_edges(torch.device("cuda"), DTYPES[dtype], 2e-4 if dtype == "float32" else 3e-2)
 
 
-@pytest.mark.parametrize("rank,rot,heads", [(64, 32, 3), (128, 64, 5), (256, 32, 70), (512, 64, 2)])
+@pytest.mark.parametrize("rank,rot,heads", [(64, 32, 3), (128, 64, 5), (256, 32, 70), (512, 64, 2),
+                                            (32, 64, 3), (64, 96, 2), (64, 128, 4), (128, 128, 2), (128, 192, 3)])
 @pytest.mark.parametrize("mode,splits", [("tiles", 1), ("decode", 1), ("decode", 3), ("decode", 7)])
 def test_attention_edges_matrix_cores(rank, rot, heads, mode, splits):
     """The tile kernel: one-token tiles and decode rows, whole key range and key-range splits (more splits
@@ -208,6 +209,37 @@ def test_tile_kernel_in_the_engine(model_c):
     zc.check_cuts("cuda", "bfloat16", tol, *model_c, 200, [[200], [], [130], [2, 2, 60, 1, 2, 61, 3, 64, 2], [63, 2, 63, 2]])
     zc.check_batches("cuda", "bfloat16", tol, *model_c)
     zc.check_cuts("cuda", "float32", 5e-5, *model_c, 150, [[150], [70, 3, 64]])
+
+
+def test_expanded_prefill_in_the_engine():
+    """Prefill parts large enough to expand keys and values per head for the step (bf16): whole prompts, a
+    second large portion over a cached first one, large portions beside decoding requests; the small portions
+    and the decoded tokens of the same requests stay in latent space and must agree with them."""
+    from vllm_production_stack_amd.models import zururax
+
+    cfg = zo.config_d()
+    w = zo.make_weights(cfg, seed=6)
+    n = 700
+    toks = zc.tokens(cfg, n, 8)
+    want = zo.forward(cfg, w, toks)
+    eng = zc.make_engine(cfg, w, "cuda", "bfloat16", pages=24)
+    assert all(eng.runner.model._expands(s.mixer) for s in eng.runner.model.specs)
+    seen = []
+    real = eng.runner.model._expanded_prefill
+    eng.runner.model._expanded_prefill = lambda *a, **k: (seen.append(a[1].shape[0]), real(*a, **k))[1]
+    for k, cuts in enumerate([[n], [300, 400], [256, 100, 300, 2, 42], [n - 40]]):
+        zo.check_rows(zc.replay(eng, f"r{k}", toks, cuts), want, 6e-2, f"cuts {cuts}")
+    assert sorted(set(seen)) == [256, 300, 400, 660, 700]  # 100, 2, 42 and single tokens stayed in latent space
+    # a large portion beside two decoding requests and a small portion
+    a, b = zc.tokens(cfg, 90, 1), zc.tokens(cfg, 40, 2)
+    la, lb = zo.forward(cfg, w, a), zo.forward(cfg, w, b)
+    eng.forced_step([("a", a[:89], []), ("b", b[:39], [])])
+    out = eng.forced_step([("a", a[89:], [0]), ("b", b[39:], [0]), ("c", toks[:500], list(range(500))), ("d", b[:7], [6])],
+                          ["a", "b", "c", "d"]).cpu()
+    zo.check_rows(out[2:502], want[:500], 6e-2, "large portion in a mixed batch")
+    zo.check_rows(torch.stack([out[0], out[1], out[502]]), torch.stack([la[89], lb[39], lb[6]]), 1e-1, "its neighbours")
+    assert zururax.EXPAND_MIN_ROWS == 256
+    eng.shutdown()
 
 
 @pytest.mark.parametrize("dtype,tol", MODES)

@@ -193,6 +193,15 @@ def config_c():
     ], embedding_scale=1.5)
 
 
+def config_d():
+    """Heads whose value | key sizes (64 | 64 + 32, 64 | 96 + 32) the tile kernel also takes as expanded
+    per-head entries (large prefill parts), the second layer reading the first one's entries."""
+    return make_config(71, 64, [
+        layer(mixer(3, 64, 32, 64, 64, 24, base=700.0), {"kind": "dense", "ff": 96}),
+        layer(mixer(2, 96, 32, 64, 64, 32, base=700.0, kv_from=0), None),
+    ], embedding_scale=1.3)
+
+
 def make_weights(cfg, seed=0, sink_std=1.0):
     """bf16-representable float64 weights (what a bf16 checkpoint holds), activations of order one."""
     g = torch.Generator().manual_seed(seed)

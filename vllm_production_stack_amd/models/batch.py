@@ -32,6 +32,7 @@ class BatchMeta:
     pre_tile_q0: torch.Tensor | None = None
     pre_tile_rows: int | None = None  # tile height the work list was built for
     pre_row_seq: torch.Tensor | None = None  # int32 [prefill rows]: the row's sequence (row-wise attention kernels)
+    pre_expand: dict | None = None  # heads -> layout and work list of a step's per-head expanded entries
     pre_lat_tiles: dict | None = None  # heads -> int32 [tiles, 6]: work lists of the latent-attention tile kernel
     # key-range splits of a short work list (ops.plan_prefill_splits): int32 [entries, 3], the fp32
     # workspace of the partial records, int32 [groups, 4]; None = every entry walks all its keys

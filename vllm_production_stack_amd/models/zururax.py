@@ -29,13 +29,16 @@ from ..ops.reference import PAGE
 from ..parallel.state import get_pp, get_tp
 from .batch import BatchMeta
 
+# Prefill parts of at least this many rows expand keys and values per head for the step (below, the
+# expansion of the whole context costs more than latent space saves)
+EXPAND_MIN_ROWS = 256
 GLU_ALPHA = 1.702   # the gated units' sigmoid slope
 GLU_UP_BIAS = 1.0   # and the offset of their linear branch
 
 
 class ZururaxLayer:
     __slots__ = ("spec", "norm1", "norm2", "w_in", "dq_norm", "dkv_norm", "w_uq", "w_uk", "w_uv", "sink", "w_o",
-                 "w_up", "w_down", "router", "w13", "w2", "w_sh13", "w_sh2", "cache_offset", "cos_sin")
+                 "w_up", "w_down", "router", "w13", "w2", "w_sh13", "w_sh2", "cache_offset", "cos_sin", "w_vk")
 
     def __init__(self, spec):
         for s in self.__slots__:
@@ -150,8 +153,23 @@ class ZururaxModel:
         for lw in self.layers:
             for s in ZururaxLayer.__slots__:
                 t = getattr(lw, s)
-                if isinstance(t, torch.Tensor) and s != "cos_sin":
+                if isinstance(t, torch.Tensor) and s not in ("cos_sin", "w_vk"):
                     yield t
+
+    # derived copies (rebuilt from the weights when needed): per head [W_uv; W_uk], the matrix that
+    # expands latents into values and unrotated keys for large prefill parts
+    def packed_tensors(self):
+        for lw in self.layers:
+            if lw.w_vk is not None:
+                yield lw.w_vk
+
+    def drop_packed(self) -> None:
+        for lw in self.layers:
+            lw.w_vk = None
+
+    def _expands(self, m: LatentMixerSpec) -> bool:
+        return (self.device.type == "cuda" and self.dtype == torch.bfloat16 and m.kv_rank % 8 == 0
+                and ops.latent_mfma_supported(m.vdim, m.dim + m.rot_dim))
 
     def weight_bytes(self) -> int:
         return sum(t.numel() * t.element_size() for t in self.weight_tensors())
@@ -164,11 +182,67 @@ class ZururaxModel:
             seq.extend([i] * n)
         meta.pre_row_seq = to_dev(seq, torch.int32)
         meta.pre_lat_tiles = {}
+        meta.pre_expand = {}
+        if sum(q_lens) >= EXPAND_MIN_ROWS:
+            for heads in sorted({s.mixer.heads for s in self.specs if self._expands(s.mixer)}):
+                meta.pre_expand[heads] = self._plan_expanded(q_lens, ctx_lens, heads)
         if self.device.type == "cuda" and self.dtype == torch.bfloat16:
             for heads in sorted({s.mixer.heads for s in self.specs
                                  if ops.latent_mfma_supported(s.mixer.kv_rank, s.mixer.rot_dim)}):
                 tiles = ops.build_latent_tiles(q_lens, ctx_lens, heads)
                 meta.pre_lat_tiles[heads] = torch.from_numpy(tiles).pin_memory().to(self.device, non_blocking=True)
+
+    def _plan_expanded(self, q_lens, ctx_lens, heads: int) -> dict:
+        """Layout of a step's expanded entries (one run of pages per prefill sequence and head) and the
+        tile list over them: 64 consecutive tokens of one head per tile."""
+        import numpy as np
+
+        n_pages = [(c + PAGE - 1) // PAGE for c in ctx_lens]
+        width = max(n_pages)
+        bt = np.zeros((len(q_lens) * heads, width), dtype=np.int32)
+        parts, base, row = [], [], 0
+        total = 0
+        for i, (n, ctx, npg) in enumerate(zip(q_lens, ctx_lens, n_pages)):
+            base.append(total)
+            for h in range(heads):
+                bt[i * heads + h, :npg] = total + h * npg + np.arange(npg)
+            k = np.arange(0, n, 64, dtype=np.int64)
+            for h in range(heads):
+                parts.append(np.stack([np.full_like(k, i * heads + h), row + k, np.minimum(64, n - k), ctx - n + k,
+                                       np.full_like(k, h), np.ones_like(k)], axis=1))
+            total += heads * npg
+            row += n
+        tiles = np.concatenate(parts)
+        tiles = tiles[np.argsort(-(tiles[:, 3] + tiles[:, 2]), kind="stable")].astype(np.int32)
+        return {"n_pages": n_pages, "base": base, "total": total,
+                "bt": torch.from_numpy(bt).pin_memory().to(self.device, non_blocking=True),
+                "tiles": torch.from_numpy(tiles).pin_memory().to(self.device, non_blocking=True)}
+
+    def _expanded_prefill(self, lw: ZururaxLayer, q: torch.Tensor, pool, meta: BatchMeta, plan: dict, out: torch.Tensor):
+        """Attention of the prefill rows with keys and values expanded per head for this step: the
+        sequences' entries are gathered from the pool, one library product makes values and unrotated
+        keys of every head, and the tile kernel runs over per-head entries value | key | rotated part
+        (its first product reads zeros against the value channels).  640 / 2176 of the latent form's
+        FLOPs per query-key pair at 128 + 64 / 128 channels and rank 512."""
+        m: LatentMixerSpec = lw.spec.mixer
+        h, v, d, r, kr = m.heads, m.vdim, m.dim, m.rot_dim, m.kv_rank
+        if lw.w_vk is None:
+            lw.w_vk = torch.cat([lw.w_uv, lw.w_uk], dim=1).reshape(h * (v + d), kr).contiguous()
+        wide = v + d + r
+        view = pool[:, lw.cache_offset:lw.cache_offset + PAGE * m.entry].view(pool.shape[0], PAGE, m.entry)
+        exp = torch.empty((plan["total"], PAGE * wide), dtype=q.dtype, device=q.device)
+        for s, (npg, base) in enumerate(zip(plan["n_pages"], plan["base"])):
+            ent = view[meta.pre_block_tables[s, :npg].long()]                      # [pages, 64, entry]
+            vk = ops.linear(ent[:, :, :kr].reshape(npg * PAGE, kr), lw.w_vk)       # [keys, heads * (v + d)]
+            dst = exp[base:base + h * npg].view(h, npg, PAGE, wide)
+            dst[:, :, :, :v + d] = vk.view(npg, PAGE, h, v + d).permute(2, 0, 1, 3)
+            dst[:, :, :, v + d:] = ent[:, :, kr:].unsqueeze(0)
+        t = q.shape[0]
+        zeros = torch.zeros((1, 1, v), dtype=q.dtype, device=q.device).expand(t, h, v)
+        if not ops.latent_tile_kernel_takes(zeros, q, exp, out):
+            raise RuntimeError("expanded prefill: operands the tile kernel does not take")
+        ops.latent_attention(zeros, q, exp, 0, plan["bt"], None, meta.positions[meta.num_decode:], lw.sink, m.scale,
+                             out=out, tiles=plan["tiles"])
 
     # ------------------------------------------------------------------ forward
     def _mixer(self, lw: ZururaxLayer, h: torch.Tensor, pool, meta: BatchMeta) -> torch.Tensor:
@@ -184,11 +258,25 @@ class ZururaxModel:
             ops.latent_kv_write(proj[:, col:col + m.entry], lw.dkv_norm, meta.positions, meta.slots, lw.cos_sin, pool,
                                 lw.cache_offset, m.kv_rank, m.rot_dim, m.rope_dims, eps)
             col += m.entry
+        nd = meta.num_decode
+        plan = (getattr(meta, "pre_expand", None) or {}).get(m.heads) if self._expands(m) else None
+        if plan is not None and meta.num_prefill_seqs > 0:
+            # large prefill part: per-head keys and values for this step; decode rows stay in latent space
+            o = torch.empty((t, m.heads, m.vdim), dtype=h.dtype, device=h.device)
+            self._expanded_prefill(lw, q[nd:], pool, meta, plan, o[nd:])
+            if nd > 0:
+                q_lat = torch.bmm(q[:nd, :, :m.dim].transpose(0, 1), lw.w_uk).transpose(0, 1)
+                o_lat = ops.latent_attention(q_lat, q[:nd, :, m.dim:], pool, lw.cache_offset, meta.dec_block_tables, None,
+                                             meta.positions[:nd], lw.sink, m.scale,
+                                             splits=getattr(meta, "dec_num_splits", 1) or 1)
+                o[:nd] = torch.bmm(o_lat.transpose(0, 1), lw.w_uv.transpose(1, 2)).transpose(0, 1)
+            if m.out_gate:
+                ops.sigmoid_gate(o, proj[:, col:col + m.heads])
+            return ops.linear(o.view(t, m.heads * m.vdim), lw.w_o)
         # [heads, T, dim] x [heads, dim, kv_rank]: the unrotated query in latent space
         q_lat = torch.bmm(q[:, :, :m.dim].transpose(0, 1), lw.w_uk).transpose(0, 1)
         q_rot = q[:, :, m.dim:]
         o_lat = torch.empty((t, m.heads, m.kv_rank), dtype=h.dtype, device=h.device)
-        nd = meta.num_decode
         if nd > 0:
             ops.latent_attention(q_lat[:nd], q_rot[:nd], pool, lw.cache_offset, meta.dec_block_tables, None,
                                  meta.positions[:nd], lw.sink, m.scale, out=o_lat[:nd],

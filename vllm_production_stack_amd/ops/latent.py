@@ -169,6 +169,11 @@ def _mfma_ok(q_lat, q_rot, pool, out) -> bool:
             and out.stride(0) % 4 == 0 and out.stride(1) % 4 == 0 and pool.stride(0) % 8 == 0)
 
 
+def latent_tile_kernel_takes(q_lat, q_rot, pool, out) -> bool:
+    """Would ``latent_attention`` run these operands on the matrix-core tile kernel?"""
+    return bool(q_lat.is_cuda and _mfma_ok(q_lat, q_rot, pool, out))
+
+
 def latent_attention(q_lat, q_rot, pool, offset: int, block_tables, row_seq, positions, sink, scale: float, out=None,
                      tiles=None, splits: int = 1):
     """Causal attention of query rows over their sequences' cache entries, in latent space.
