@@ -11,7 +11,10 @@ rotated key part shared by all heads (``kv_rank + rot_dim`` values; layers with 
 entries of the layer they name and own no cache).  Keys and values are never expanded: a head's
 unrotated query is carried into latent space (q W_uk, one batched matrix product), the attention
 kernel scores it against the entries and returns the probability-weighted latent, and W_uv takes
-that to the head's value space.  All heads then share one key/value stream per token.
+that to the head's value space.  All heads then share one key/value stream per token.  Large prefill
+parts (``EXPAND_MIN_ROWS``) are the exception: there the 3.4 x FLOPs of latent space outweigh what it
+saves, so values and unrotated keys of every head are expanded for the step (one library product over
+the sequences' gathered entries) and the same tile kernel runs over per-head entries.
 
 The input projections of a mixer (query latent | KV latent and shared key part | output-gate logits)
 are one fused matrix, as are gate | up of every gated unit; the router's matrix (with the shared
