@@ -114,7 +114,10 @@ def build_target(name: str, force: bool = False) -> Path | None:
     else:
         cmd = [CXX, "-O2", "-std=c++17", *shared, "-I", str(CSRC), *map(str, paths), "-o",
                str(out), *flags]
-    _run(cmd)
+    # link under a temporary name: a build that is cut short never leaves half a library where loaders look
+    tmp = out.with_name(out.name + ".part")
+    _run([str(tmp) if c == str(out) else c for c in cmd])
+    os.replace(tmp, out)
     return out
 
 
