@@ -1,0 +1,510 @@
+// Sequence mixers with carried state, for gfx950: linear-attention recurrences (fixed decay per head, or a
+// forget gate per channel that also decides what is written), a short causal convolution in front of a
+// windowed softmax attention with kept first tokens, capped scores, a sink and post-softmax head mixing,
+// the Dynamic Tanh norm on a 32-bit residual stream, and the xIELU activation.  bf16 or fp32 activations
+// (dtype 0 / 1 in the entry points); norms, angles, gates, decays, recurrent state, scores and softmax
+// weights are fp32 in both.
+//
+//   add_dyt            residual += s1 d1 + s2 d2;  y = tanh(alpha residual) w + b
+//   recurrent_scan     per (sequence, head): S <- a_t (.) S + k_t v_t^T,  o_t = S^T q_t, state in registers,
+//                      carried in a per-sequence fp32 slot (zero when the chunk starts at position 0)
+//   head_rms           o[t, h, :] / rms(o[t, h, :]) (* w) (* silu(gate[t, h, :]))
+//   short_conv_qkv     y_t = sum_j w[:, j] u_(t - taps + 1 + j) over a sequence's projected rows (the rows
+//                      before the chunk come from the sequence's slot), rotary q / k, k and v -> paged cache
+//   conv_tail          the last taps - 1 projected rows of every sequence -> its slot
+//   window_attention   softmax(cap tanh(q k scale / cap)) with a sink in the denominator over the keys
+//                      j <= i with i - j < window or j < keep_first, applied to the values of EVERY KV head
+//   mix_heads          out[t, h] = sum_g talk[h, g] u[t, g, kv_head(h)]
+//   xielu              z > 0: a_p z^2 + z / 2;  else a_n (exp(z) - 1 - z) + z / 2
+//
+// Plain kernels: every size is taken (bounds below are checked by the entry points).
+#include "common.h"
+
+namespace {
+
+template <typename T> struct Cv;
+template <> struct Cv<float> {
+  static __device__ __forceinline__ float ld(const float* p) { return *p; }
+  static __device__ __forceinline__ void st(float* p, float v) { *p = v; }
+  static __device__ __forceinline__ float round(float v) { return v; }
+};
+template <> struct Cv<bf16_t> {
+  static __device__ __forceinline__ float ld(const bf16_t* p) { return (float)*p; }
+  static __device__ __forceinline__ void st(bf16_t* p, float v) { *p = (bf16_t)v; }
+  static __device__ __forceinline__ float round(float v) { return (float)(bf16_t)v; }
+};
+
+__device__ __forceinline__ float blk_sum(float v, float* red) {
+  v = wave_reduce_sum(v);
+  const int tid = threadIdx.x;
+  __syncthreads();
+  if ((tid & 63) == 0) red[tid >> 6] = v;
+  __syncthreads();
+  float s = 0.f;
+  for (int i = 0; i < (int)(blockDim.x >> 6); ++i) s += red[i];
+  return s;
+}
+
+__device__ __forceinline__ float blk_max(float v, float* red) {
+  v = wave_reduce_max(v);
+  const int tid = threadIdx.x;
+  __syncthreads();
+  if ((tid & 63) == 0) red[tid >> 6] = v;
+  __syncthreads();
+  float s = red[0];
+  for (int i = 1; i < (int)(blockDim.x >> 6); ++i) s = fmaxf(s, red[i]);
+  return s;
+}
+
+__device__ __forceinline__ float sigm(float x) { return 1.f / (1.f + expf(-x)); }
+
+// Channel i of a head after the rotation of its first `dims` channels; x(c) reads channel c, cs is the
+// table row of the token's position (cos[0 .. dims/2) | sin[0 .. dims/2)).  layout 0 pairs channel c with
+// c + dims/2, layout 1 pairs 2c with 2c + 1.
+template <typename F>
+__device__ __forceinline__ float rotated(F x, int i, const float* __restrict__ cs, int dims, int layout) {
+  if (i >= dims) return x(i);
+  const int half = dims >> 1;
+  if (layout == 0) {
+    if (i < half) return x(i) * cs[i] - x(i + half) * cs[half + i];
+    return x(i) * cs[i - half] + x(i - half) * cs[i];
+  }
+  const int p = i >> 1;
+  if ((i & 1) == 0) return x(i) * cs[p] - x(i + 1) * cs[half + p];
+  return x(i) * cs[p] + x(i - 1) * cs[half + p];
+}
+
+// ---------------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void add_dyt_kernel(float* __restrict__ residual, const T* __restrict__ d1, long s1,
+                                                      float c1, const T* __restrict__ d2, long s2, float c2,
+                                                      const float* __restrict__ w, const float* __restrict__ b,
+                                                      const float* __restrict__ alpha, T* __restrict__ y, int n) {
+  const long row = blockIdx.x;
+  float* r = residual + row * n;
+  const float a = alpha[0];
+  for (int i = threadIdx.x; i < n; i += 256) {
+    float v = r[i];
+    if (d1) v += c1 * Cv<T>::ld(d1 + row * s1 + i);
+    if (d2) v += c2 * Cv<T>::ld(d2 + row * s2 + i);
+    if (d1 || d2) r[i] = v;
+    if (y) Cv<T>::st(y + row * (long)n + i, tanhf(a * v) * w[i] + b[i]);
+  }
+}
+
+// ---------------------------------------------------------------------------------
+// One workgroup = 256 / R state columns of one head of one sequence; a state column's `dim` rows are
+// spread over R neighbouring lanes, RPT rows each (row i = j * R + lane group), all in registers.
+// A block of up to TB tokens is prepared in LDS (rotation or gates, fp32), then walked token by token.
+template <typename T, int RPT, bool GATED>
+__global__ __launch_bounds__(256) void recurrent_scan_kernel(
+    const T* __restrict__ proj, long p_stride, int q_col, int k_col, int v_col, int heads, int dim, int vdim,
+    float* __restrict__ state, long state_stride, const int* __restrict__ seq_cu, const int* __restrict__ seq_state,
+    const int* __restrict__ positions, const float* __restrict__ decay, const float* __restrict__ cos_sin, int rot_dims,
+    int layout, float k_scale, const float* __restrict__ gate_bias, const float* __restrict__ gate_lower,
+    float* __restrict__ out, int R, int TB) {
+  extern __shared__ float smem[];
+  const int seq = blockIdx.z, head = blockIdx.y;
+  const int slot = seq_state[seq];
+  const int r0 = seq_cu[seq], r1 = seq_cu[seq + 1];
+  const int dimp = R * RPT, cols = 256 / R;
+  if (slot < 0) {  // rows of no sequence (a padded batch): their output is zero
+    for (int e = threadIdx.x; e < (r1 - r0) * cols; e += 256) {
+      const int c = blockIdx.x * cols + e % cols;
+      if (c < vdim) out[((long)(r0 + e / cols) * heads + head) * vdim + c] = 0.f;
+    }
+    return;
+  }
+  if (r1 <= r0) return;
+  float* qs = smem;
+  float* ks = qs + TB * dimp;
+  float* as = ks + TB * dimp;                       // gates (GATED only)
+  float* vs = GATED ? as + TB * dimp : as;
+  const int tid = threadIdx.x, rg = tid % R, cb = tid / R;
+  const int col = blockIdx.x * cols + cb;
+  const bool colok = col < vdim;
+  float* st = state + (long)slot * state_stride + (long)head * dim * vdim;
+  const bool fresh = positions[r0] == 0;
+  float S[RPT];
+#pragma unroll
+  for (int j = 0; j < RPT; ++j) {
+    const int i = j * R + rg;
+    S[j] = (!fresh && colok && i < dim) ? st[(long)i * vdim + col] : 0.f;
+  }
+  const float dec = GATED ? 0.f : decay[head];
+  for (int rb = r0; rb < r1; rb += TB) {
+    const int nb = min(TB, r1 - rb);
+    __syncthreads();
+    for (int e = tid; e < nb * dimp; e += 256) {
+      const int tt = e / dimp, i = e - tt * dimp;
+      const long row = rb + tt;
+      float q = 0.f, k = 0.f, a = 0.f;
+      if (i < dim) {
+        const T* qp = proj + row * p_stride + q_col + head * dim;
+        const T* kp = proj + row * p_stride + k_col + head * dim;
+        if (GATED) {
+          const float x = Cv<T>::ld(qp + i);
+          q = x * sigm(x);
+          const float lo = gate_lower[head * dim + i];
+          a = lo + (1.f - lo) * sigm(Cv<T>::ld(kp + i) + gate_bias[head * dim + i]);
+          k = 1.f - a;
+        } else {
+          const float* cs = cos_sin + (long)positions[row] * rot_dims;
+          q = rotated([&](int c) { return Cv<T>::ld(qp + c); }, i, cs, rot_dims, layout);
+          k = rotated([&](int c) { return Cv<T>::ld(kp + c); }, i, cs, rot_dims, layout) * k_scale;
+        }
+      }
+      qs[e] = q;
+      ks[e] = k;
+      if (GATED) as[e] = a;
+    }
+    for (int e = tid; e < nb * cols; e += 256) {
+      const int tt = e / cols, c = e - tt * cols;
+      const int cc = blockIdx.x * cols + c;
+      vs[e] = cc < vdim ? Cv<T>::ld(proj + (long)(rb + tt) * p_stride + v_col + head * vdim + cc) : 0.f;
+    }
+    __syncthreads();
+    for (int tt = 0; tt < nb; ++tt) {
+      const float v = vs[tt * cols + cb];
+      const float* qr = qs + tt * dimp + rg;
+      const float* kr = ks + tt * dimp + rg;
+      const float* ar = as + tt * dimp + rg;
+      float acc = 0.f;
+#pragma unroll
+      for (int j = 0; j < RPT; ++j) {
+        const float kv = kr[j * R] * v;
+        S[j] = GATED ? fmaf(ar[j * R], S[j], kv) : fmaf(dec, S[j], kv);
+        acc = fmaf(S[j], qr[j * R], acc);
+      }
+      for (int off = R >> 1; off > 0; off >>= 1) acc += __shfl_xor(acc, off, 64);
+      if (rg == 0 && colok) out[((long)(rb + tt) * heads + head) * vdim + col] = acc;
+    }
+  }
+  if (colok) {
+#pragma unroll
+    for (int j = 0; j < RPT; ++j) {
+      const int i = j * R + rg;
+      if (i < dim) st[(long)i * vdim + col] = S[j];
+    }
+  }
+}
+
+// one wave per (row, head)
+template <typename T>
+__global__ __launch_bounds__(256) void head_rms_kernel(const float* __restrict__ o, const float* __restrict__ w,
+                                                       const T* __restrict__ gate, long g_stride, T* __restrict__ y,
+                                                       long pairs, int heads, int vdim, float eps) {
+  const long pair = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (pair >= pairs) return;
+  const int lane = threadIdx.x & 63;
+  const long row = pair / heads;
+  const int head = (int)(pair - row * heads);
+  const float* op = o + pair * vdim;
+  float ss = 0.f;
+  for (int c = lane; c < vdim; c += 64) ss += op[c] * op[c];
+  ss = wave_reduce_sum(ss);
+  const float inv = 1.f / sqrtf(ss / (float)vdim + eps);
+  for (int c = lane; c < vdim; c += 64) {
+    float v = op[c] * inv;
+    if (w) v *= w[c];
+    if (gate) {
+      const float g = Cv<T>::ld(gate + row * g_stride + head * vdim + c);
+      v *= g * sigm(g);
+    }
+    Cv<T>::st(y + pair * vdim + c, v);
+  }
+}
+
+// ---------------------------------------------------------------------------------
+// One workgroup per row.  chans = heads * dim + kv_heads * (dim + vdim) projected channels q | k | v.
+template <typename T>
+__global__ __launch_bounds__(256) void short_conv_qkv_kernel(
+    const T* __restrict__ proj, long p_stride, const float* __restrict__ conv_w, int taps, int heads, int kv_heads,
+    int dim, int vdim, const float* __restrict__ state, long state_stride, const int* __restrict__ row_seq,
+    const int* __restrict__ seq_cu, const int* __restrict__ seq_state, const int* __restrict__ positions,
+    const long* __restrict__ slots, const float* __restrict__ cos_sin, int rot_dims, int layout, T* __restrict__ q_out,
+    T* __restrict__ cache, long page_stride) {
+  extern __shared__ float ys[];
+  const long row = blockIdx.x;
+  const int seq = row_seq ? row_seq[row] : (int)row;
+  const int slot = seq_state[seq];
+  const int r0 = seq_cu[seq];
+  const int pos = positions[row], pos0 = positions[r0];
+  const int chans = heads * dim + kv_heads * (dim + vdim);
+  const float* tail = slot >= 0 ? state + (long)slot * state_stride : nullptr;
+  for (int c = threadIdx.x; c < chans; c += 256) {
+    float acc = 0.f;
+    for (int j = 0; j < taps; ++j) {
+      const int back = taps - 1 - j;
+      const long src = row - back;
+      float u = 0.f;
+      if (src >= r0) {
+        u = Cv<T>::ld(proj + src * p_stride + c);
+      } else if (pos - back >= 0 && tail) {
+        u = tail[(long)(pos - back - (pos0 - (taps - 1))) * chans + c];
+      }
+      acc = fmaf(conv_w[(long)c * taps + j], u, acc);
+    }
+    ys[c] = Cv<T>::round(acc);
+  }
+  __syncthreads();
+  const float* cs = cos_sin + (long)pos * rot_dims;
+  const int nq = heads * dim, nk = kv_heads * dim, nv = kv_heads * vdim;
+  const long kv_slot = slots[row];
+  T* kdst = kv_slot >= 0 ? cache + (kv_slot / PAGE) * page_stride + (kv_slot % PAGE) * (long)nk : nullptr;
+  T* vdst = kv_slot >= 0 ? cache + (kv_slot / PAGE) * page_stride + (long)PAGE * nk + (kv_slot % PAGE) * (long)nv : nullptr;
+  for (int c = threadIdx.x; c < chans; c += 256) {
+    if (c < nq + nk) {
+      const int base = c < nq ? (c / dim) * dim : nq + ((c - nq) / dim) * dim;
+      const float* x = ys + base;
+      const float r = rotated([&](int i) { return x[i]; }, c - base, cs, rot_dims, layout);
+      if (c < nq) Cv<T>::st(q_out + row * nq + c, r);
+      else if (kdst) Cv<T>::st(kdst + (c - nq), r);
+    } else if (vdst) {
+      Cv<T>::st(vdst + (c - nq - nk), ys[c]);
+    }
+  }
+}
+
+// One workgroup per sequence, after the convolution of the step: tail[j] = projected row of position
+// end - (taps - 1) + j, from the chunk or, for chunks shorter than the tail, from the old tail (shifted:
+// a thread owns a channel and walks j upwards, so it reads tail[j + n] before writing it).
+template <typename T>
+__global__ __launch_bounds__(256) void conv_tail_kernel(const T* __restrict__ proj, long p_stride, int taps, int chans,
+                                                        float* __restrict__ state, long state_stride,
+                                                        const int* __restrict__ seq_cu, const int* __restrict__ seq_state,
+                                                        const int* __restrict__ positions) {
+  const int seq = blockIdx.x;
+  const int slot = seq_state[seq];
+  const int r0 = seq_cu[seq], r1 = seq_cu[seq + 1];
+  if (slot < 0 || r1 <= r0) return;
+  const int n = r1 - r0, pos0 = positions[r0], keep = taps - 1;
+  float* tail = state + (long)slot * state_stride;
+  for (int c = threadIdx.x; c < chans; c += 256) {
+    for (int j = 0; j < keep; ++j) {
+      const int k = n + j - keep;  // chunk row of tail entry j (negative: before the chunk)
+      float u = 0.f;
+      if (k >= 0) u = Cv<T>::ld(proj + (long)(r0 + k) * p_stride + c);
+      else if (pos0 + k >= 0) u = tail[(long)(j + n) * chans + c];
+      tail[(long)j * chans + c] = u;
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------
+// One workgroup per (row, query head): 256 keys per step.  Layer cache inside a page: K [PAGE][kv_heads * dim],
+// then V [PAGE][kv_heads * vdim].  out [rows, heads, kv_heads, vdim] fp32: the head's softmax weights applied
+// to the values of every KV head (the head mixing that follows needs them).
+constexpr int WA_KEYS = 256;
+constexpr int WA_ACC = 8;  // kv_heads * vdim <= 256 * WA_ACC
+
+template <typename T>
+__global__ __launch_bounds__(256) void window_attention_kernel(
+    const T* __restrict__ q, long q_stride, const T* __restrict__ cache, long page_stride,
+    const int* __restrict__ block_tables, int bt_stride, const int* __restrict__ row_seq,
+    const int* __restrict__ positions, const float* __restrict__ sink, float* __restrict__ out, int heads, int kv_heads,
+    int dim, int vdim, int window, int keep_first, float scale, float softcap) {
+  extern __shared__ float sm[];
+  __shared__ float red[4];
+  __shared__ float ps[WA_KEYS];
+  __shared__ long voff[WA_KEYS];
+  const long row = blockIdx.x;
+  const int head = blockIdx.y;
+  const int tid = threadIdx.x;
+  const int seq = row_seq ? row_seq[row] : (int)row;
+  const int pos = positions[row];
+  const int g = head / (heads / kv_heads);
+  const int nk = kv_heads * dim, nv = kv_heads * vdim;
+  float* qs = sm;
+  for (int i = tid; i < dim; i += 256) qs[i] = Cv<T>::ld(q + row * q_stride + head * dim + i);
+  const int lo = max(0, pos - window + 1);
+  const int nkeep = min(keep_first, lo);
+  const int total = nkeep + (pos - lo + 1);
+  const int* bt = block_tables + (long)seq * bt_stride;
+  float m = sink ? sink[head] : -INFINITY, l = sink ? 1.f : 0.f;
+  float acc[WA_ACC];
+#pragma unroll
+  for (int a = 0; a < WA_ACC; ++a) acc[a] = 0.f;
+  __syncthreads();
+  for (int k0 = 0; k0 < total; k0 += WA_KEYS) {
+    const int kk = k0 + tid;
+    float s = -INFINITY;
+    long off = 0;
+    if (kk < total) {
+      const int j = kk < nkeep ? kk : lo + (kk - nkeep);
+      const long page = (long)bt[j / PAGE] * page_stride;
+      off = page + (long)PAGE * nk + (long)(j % PAGE) * nv;  // the key's value row
+      const T* kp = cache + page + (long)(j % PAGE) * nk + g * dim;
+      float d = 0.f;
+      for (int i = 0; i < dim; ++i) d = fmaf(qs[i], Cv<T>::ld(kp + i), d);
+      d *= scale;
+      s = softcap > 0.f ? softcap * tanhf(d / softcap) : d;
+    }
+    const float mb = blk_max(s, red);
+    const float mn = fmaxf(m, mb);
+    const float p = kk < total ? expf(s - mn) : 0.f;
+    const float corr = expf(m - mn);  // 0 while nothing has been seen (m = -inf without a sink)
+    ps[tid] = p;
+    voff[tid] = off;
+    const float bs = blk_sum(p, red);  // its barriers also publish ps / voff
+    l = l * corr + bs;
+    const int nb = min(WA_KEYS, total - k0);
+#pragma unroll
+    for (int a = 0; a < WA_ACC; ++a) {
+      const int c = a * 256 + tid;
+      if (c < nv) {
+        float x = acc[a] * corr;
+        for (int k = 0; k < nb; ++k) x = fmaf(ps[k], Cv<T>::ld(cache + voff[k] + c), x);
+        acc[a] = x;
+      }
+    }
+    m = mn;
+    __syncthreads();
+  }
+  const float inv = 1.f / l;
+#pragma unroll
+  for (int a = 0; a < WA_ACC; ++a) {
+    const int c = a * 256 + tid;
+    if (c < nv) out[(row * heads + head) * (long)nv + c] = acc[a] * inv;
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void mix_heads_kernel(const float* __restrict__ u, const float* __restrict__ talk,
+                                                        T* __restrict__ y, int heads, int kv_heads, int vdim) {
+  const long row = blockIdx.x;
+  const int rep = heads / kv_heads;
+  const float* ur = u + row * (long)heads * kv_heads * vdim;
+  for (int e = threadIdx.x; e < heads * vdim; e += 256) {
+    const int h = e / vdim, c = e - h * vdim;
+    const int own = h / rep;
+    float acc = 0.f;
+    for (int g = 0; g < heads; ++g) acc = fmaf(talk[h * heads + g], ur[((long)g * kv_heads + own) * vdim + c], acc);
+    Cv<T>::st(y + row * (long)heads * vdim + e, acc);
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void xielu_kernel(const T* __restrict__ x, T* __restrict__ y, long n,
+                                                    const float* __restrict__ act) {
+  const float ap = act[0], an = act[1];
+  for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long)gridDim.x * 256) {
+    const float z = Cv<T>::ld(x + i);
+    const float v = z > 0.f ? fmaf(ap * z, z, 0.5f * z) : fmaf(an, expm1f(z) - z, 0.5f * z);
+    Cv<T>::st(y + i, v);
+  }
+}
+
+}  // namespace
+
+#define SM_DISPATCH(dt, CALL)                         \
+  if ((dt) == 0) { using T = bf16_t; CALL; }          \
+  else if ((dt) == 1) { using T = float; CALL; }      \
+  else return 1;
+
+VPSA_EXPORT int vpsa_add_dyt(float* residual, const void* d1, long s1, float c1, const void* d2, long s2, float c2,
+                             const float* w, const float* b, const float* alpha, void* y, int rows, int n, int dt,
+                             hipStream_t stream) {
+  if (rows <= 0) return 0;
+  SM_DISPATCH(dt, (add_dyt_kernel<T><<<rows, 256, 0, stream>>>(residual, (const T*)d1, s1, c1, (const T*)d2, s2, c2, w, b,
+                                                               alpha, (T*)y, n)));
+  return 0;
+}
+
+// Rows of the state a lane holds and lanes per state column for a head of `dim` rows.
+static void scan_shape(int dim, int* rpt, int* r) {
+  for (int p = 8;; p <<= 1) {
+    int lanes = 1;
+    while (lanes * p < dim) lanes <<= 1;
+    if (lanes <= 4 || p == 32) { *rpt = p; *r = lanes; return; }
+  }
+}
+
+VPSA_EXPORT int vpsa_recurrent_scan(const void* proj, long p_stride, int q_col, int k_col, int v_col, int heads, int dim,
+                                    int vdim, float* state, long state_stride, const int* seq_cu, const int* seq_state,
+                                    int n_seqs, const int* positions, const float* decay, const float* cos_sin,
+                                    int rot_dims, int layout, float k_scale, const float* gate_bias,
+                                    const float* gate_lower, float* out, int gated, int dt, hipStream_t stream) {
+  if (n_seqs <= 0) return 0;
+  int rpt, r;
+  scan_shape(dim, &rpt, &r);
+  if (r > 64) return 2;
+  const int dimp = r * rpt, cols = 256 / r;
+  const int per_tok = (gated ? 3 : 2) * dimp + cols;
+  int tb = (48 * 1024 / 4) / per_tok;
+  if (tb > 16) tb = 16;
+  if (tb < 1) return 3;
+  const size_t lds = (size_t)tb * per_tok * sizeof(float);
+  dim3 grid((vdim + cols - 1) / cols, heads, n_seqs);
+#define SCAN(RPT, G)                                                                                                   \
+  recurrent_scan_kernel<T, RPT, G><<<grid, 256, lds, stream>>>((const T*)proj, p_stride, q_col, k_col, v_col, heads,   \
+                                                               dim, vdim, state, state_stride, seq_cu, seq_state,      \
+                                                               positions, decay, cos_sin, rot_dims, layout, k_scale,   \
+                                                               gate_bias, gate_lower, out, r, tb)
+#define SCAN_R(G)                                  \
+  if (rpt == 8) SCAN(8, G);                        \
+  else if (rpt == 16) SCAN(16, G);                 \
+  else SCAN(32, G);
+  if (gated) { SM_DISPATCH(dt, SCAN_R(true)); }
+  else { SM_DISPATCH(dt, SCAN_R(false)); }
+#undef SCAN
+#undef SCAN_R
+  return 0;
+}
+
+VPSA_EXPORT int vpsa_head_rms(const float* o, const float* w, const void* gate, long g_stride, void* y, int rows,
+                              int heads, int vdim, float eps, int dt, hipStream_t stream) {
+  const long pairs = (long)rows * heads;
+  if (pairs <= 0) return 0;
+  SM_DISPATCH(dt, (head_rms_kernel<T><<<(unsigned)((pairs + 3) / 4), 256, 0, stream>>>(o, w, (const T*)gate, g_stride,
+                                                                                       (T*)y, pairs, heads, vdim, eps)));
+  return 0;
+}
+
+VPSA_EXPORT int vpsa_short_conv_qkv(const void* proj, long p_stride, const float* conv_w, int taps, int heads,
+                                    int kv_heads, int dim, int vdim, float* state, long state_stride,
+                                    const int* row_seq, const int* seq_cu, const int* seq_state, int n_seqs,
+                                    const int* positions, const long* slots, const float* cos_sin, int rot_dims,
+                                    int layout, void* q_out, void* cache, long page_stride, int rows, int dt,
+                                    hipStream_t stream) {
+  if (rows <= 0) return 0;
+  const int chans = heads * dim + kv_heads * (dim + vdim);
+  if ((size_t)chans * 4 > 60 * 1024 || taps < 1) return 2;
+  SM_DISPATCH(dt, (short_conv_qkv_kernel<T><<<rows, 256, (size_t)chans * 4, stream>>>(
+                      (const T*)proj, p_stride, conv_w, taps, heads, kv_heads, dim, vdim, state, state_stride, row_seq,
+                      seq_cu, seq_state, positions, slots, cos_sin, rot_dims, layout, (T*)q_out, (T*)cache, page_stride)));
+  if (taps > 1) {
+    SM_DISPATCH(dt, (conv_tail_kernel<T><<<n_seqs, 256, 0, stream>>>((const T*)proj, p_stride, taps, chans, state,
+                                                                     state_stride, seq_cu, seq_state, positions)));
+  }
+  return 0;
+}
+
+VPSA_EXPORT int vpsa_window_attention(const void* q, long q_stride, const void* cache, long page_stride,
+                                      const int* block_tables, int bt_stride, const int* row_seq, const int* positions,
+                                      const float* sink, float* out, int rows, int heads, int kv_heads, int dim, int vdim,
+                                      int window, int keep_first, float scale, float softcap, int dt,
+                                      hipStream_t stream) {
+  if (rows <= 0) return 0;
+  if (kv_heads * vdim > 256 * WA_ACC || (size_t)dim * 4 > 32 * 1024) return 2;
+  dim3 grid(rows, heads);
+  SM_DISPATCH(dt, (window_attention_kernel<T><<<grid, 256, (size_t)dim * 4, stream>>>(
+                      (const T*)q, q_stride, (const T*)cache, page_stride, block_tables, bt_stride, row_seq, positions,
+                      sink, out, heads, kv_heads, dim, vdim, window, keep_first, scale, softcap)));
+  return 0;
+}
+
+VPSA_EXPORT int vpsa_mix_heads(const float* u, const float* talk, void* y, int rows, int heads, int kv_heads, int vdim,
+                               int dt, hipStream_t stream) {
+  if (rows <= 0) return 0;
+  SM_DISPATCH(dt, (mix_heads_kernel<T><<<rows, 256, 0, stream>>>(u, talk, (T*)y, heads, kv_heads, vdim)));
+  return 0;
+}
+
+VPSA_EXPORT int vpsa_xielu(const void* x, void* y, long n, const float* act, int dt, hipStream_t stream) {
+  if (n <= 0) return 0;
+  long blocks = (n + 255) / 256;
+  if (blocks > 65536) blocks = 65536;
+  SM_DISPATCH(dt, (xielu_kernel<T><<<(unsigned)blocks, 256, 0, stream>>>((const T*)x, (T*)y, n, act)));
+  return 0;
+}

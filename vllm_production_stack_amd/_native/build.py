@@ -33,7 +33,7 @@ TARGETS = {
         ["kernels/elementwise.hip", "kernels/attention.hip", "kernels/kvcache.hip", "kernels/moe.hip",
          "kernels/lora.hip", "kernels/gemm.hip", "kernels/rans.hip", "kernels/sampling.hip",
          "kernels/grouped_gemm.hip", "kernels/packed_gemm.hip", "kernels/dense_attention.hip",
-         "kernels/tile_gemm.hip", "kernels/latent.hip", "kernels/latent_mfma.hip"],
+         "kernels/tile_gemm.hip", "kernels/latent.hip", "kernels/latent_mfma.hip", "kernels/seqmix.hip"],
         [],
     ),
     "vpsa_kvio": ("hip", ["kvio/kvio.cpp"], []),

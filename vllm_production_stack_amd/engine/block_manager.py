@@ -183,3 +183,26 @@ class BlockManager:
             self.free_ids.append(p)
             n += 1
         return n
+
+
+class StateSlots:
+    """Slots of a per-sequence state pool (models whose mixers carry state from token to token): a
+    sequence takes one when it starts running and gives it back when it finishes, is aborted or is
+    preempted (a preempted sequence is recomputed from its first token, and a chunk that starts at
+    position 0 starts from zero state: slots are never cleared)."""
+
+    def __init__(self, num_slots: int):
+        self.num_slots = num_slots
+        self.free_ids: deque[int] = deque(range(num_slots))
+
+    def num_free(self) -> int:
+        return len(self.free_ids)
+
+    def take(self) -> int:
+        if not self.free_ids:
+            raise MemoryError(f"all {self.num_slots} state slots are taken")
+        return self.free_ids.popleft()
+
+    def give_back(self, slot: int) -> None:
+        assert 0 <= slot < self.num_slots and slot not in self.free_ids
+        self.free_ids.append(slot)

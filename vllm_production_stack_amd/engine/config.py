@@ -40,14 +40,20 @@ class LatentMixerSpec:
     def entry(self) -> int:    # cached values per token
         return self.kv_rank + self.rot_dim
 
+    def weight_count(self, width: int) -> int:
+        n = width * (self.q_rank + self.heads) + self.q_rank * self.heads * (self.dim + self.rot_dim)
+        n += self.heads * self.vdim * width + self.heads * self.kv_rank * (self.dim + self.vdim)
+        return n + (width * self.entry if self.kv_from is None else 0)
+
 
 @dataclass(frozen=True)
 class FeedForwardSpec:
-    """``dense``: down(relu(up x)^2).  ``moe``: ``experts`` clamped gated units of width ``ff``, ``top``
+    """``dense``: down(act(up x)), act = relu(.)^2 unless ``act`` says otherwise.  ``moe``: ``experts`` clamped gated units of width ``ff``, ``top``
     per token out of the ``keep`` best of ``groups`` groups, sigmoid scores times ``route_scale``;
     an always-on shared unit of width ``shared_ff`` (0 = none) with a per-token sigmoid gate."""
     kind: str = "dense"
     ff: int = 0
+    act: str = "relu_sq"       # dense units: relu_sq | xielu (two learned curvatures, see ops.xielu)
     experts: int = 0
     top: int = 0
     groups: int = 1
@@ -63,6 +69,165 @@ class LayerSpec:
     type: str
     mixer: LatentMixerSpec
     mlp: FeedForwardSpec | None = None
+
+
+@dataclass(frozen=True)
+class RotarySpec:
+    """Rotary positions on the first ``dims`` channels of a head.  ``layout``: which channels form a
+    pair, ``half`` = (i, i + dims / 2), ``pairs`` = (2 i, 2 i + 1).  ``scaling`` = (factor, original,
+    fast, slow): frequencies whose wavelength exceeds the original context are divided by ``factor``
+    behind a linear ramp between the channels that make ``fast`` and ``slow`` turns over it, and cos
+    and sin carry the factor 0.1 ln(factor) + 1."""
+    base: float
+    dims: int
+    layout: str = "half"
+    scaling: tuple | None = None
+
+    def table_scaling(self) -> dict | None:
+        if self.scaling is None:
+            return None
+        factor, original, fast, slow = self.scaling
+        return {"rope_type": "ramp", "factor": factor, "original": original, "fast": fast, "slow": slow}
+
+
+@dataclass(frozen=True)
+class RetentionSpec:
+    """Linear attention with one fixed decay per head, no softmax and no denominator: per head a
+    ``dim`` x ``vdim`` state S <- decay S + k v^T, read by the rotated query; head outputs are brought
+    to unit root mean square and gated by silu(W_g h)."""
+    heads: int
+    dim: int
+    vdim: int
+    decay: tuple
+    rot: RotarySpec
+
+    def state_elems(self) -> int:
+        return self.heads * self.dim * self.vdim
+
+    def weight_count(self, width: int) -> int:
+        return width * self.heads * (2 * self.dim + 2 * self.vdim) + self.heads * self.vdim * width
+
+    def token_flops(self) -> float:      # the state update and its read-out, per token
+        return 4.0 * self.heads * self.dim * self.vdim
+
+
+@dataclass(frozen=True)
+class WindowAttentionSpec:
+    """Grouped-query softmax attention behind a short causal convolution of q, k and v: capped scores
+    (cap tanh(s / cap)), a sliding window of ``window`` positions that also keeps the first
+    ``keep_first`` tokens, a per-head sink logit in the denominator, and the heads' weights mixed by
+    an [heads, heads] matrix after the softmax."""
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    conv: int
+    window: int
+    keep_first: int
+    rot: RotarySpec
+    scale: float
+    softcap: float
+
+    @property
+    def channels(self) -> int:           # of the fused q | k | v projection
+        return self.heads * self.dim + self.kv_heads * (self.dim + self.vdim)
+
+    def state_elems(self) -> int:        # the projected rows the convolution still needs
+        return max(self.conv - 1, 0) * self.channels
+
+    def cache_elems(self) -> int:        # per token: rotated keys and values of every KV head
+        return self.kv_heads * (self.dim + self.vdim)
+
+    def weight_count(self, width: int) -> int:
+        return width * self.channels + self.heads * self.vdim * width
+
+
+@dataclass(frozen=True)
+class GatedRecurrenceSpec:
+    """Linear attention whose forget gate also decides what is written: S <- diag(f) S + (1 - f) v^T,
+    f = lower + (1 - lower) sigmoid(W_f h + b) per head and query channel; q = silu(W_q h); head
+    outputs are RMS-normed with one weight vector shared by the heads."""
+    heads: int
+    dim: int
+    vdim: int
+
+    def state_elems(self) -> int:
+        return self.heads * self.dim * self.vdim
+
+    def weight_count(self, width: int) -> int:
+        return width * self.heads * (2 * self.dim + self.vdim) + self.heads * self.vdim * width
+
+    def token_flops(self) -> float:
+        return 4.0 * self.heads * self.dim * self.vdim
+
+
+@dataclass(frozen=True)
+class ParallelMixerSpec:
+    """Two mixers that read the same input; the layer adds left_scale * left + right_scale * right."""
+    left: WindowAttentionSpec
+    right: GatedRecurrenceSpec
+    left_scale: float
+    right_scale: float
+
+    def weight_count(self, width: int) -> int:
+        return self.left.weight_count(width) + self.right.weight_count(width)
+
+
+def _rotary(rot: dict, layout: str) -> RotarySpec:
+    sc = rot.get("scaling")
+    scaling = None if not sc else (float(sc["factor"]), float(sc["original"]), float(sc["fast"]), float(sc["slow"]))
+    dims = int(rot["dims"])
+    if dims % 2:
+        raise ValueError("rotary dims must be even")
+    return RotarySpec(float(rot["base"]), dims, layout, scaling)
+
+
+def revelix_layers(layers: list[dict]) -> tuple:
+    """The ``layers`` list of a Revelix config.json -> layer specs."""
+    out = []
+    for i, entry in enumerate(layers):
+        m = entry["mixer"]
+        kind = entry["type"]
+        if kind == "retention":
+            mixer = RetentionSpec(int(m["heads"]), int(m["dim"]), int(m["vdim"]), tuple(float(d) for d in m["decay"]),
+                                  _rotary(m["rot"], "half"))
+            if len(mixer.decay) != mixer.heads or mixer.rot.dims > mixer.dim:
+                raise ValueError(f"layer {i}: one decay per head and rotary dims within the head are required")
+        elif kind == "parallel":
+            a, r = m["left"], m["right"]
+            left = WindowAttentionSpec(
+                heads=int(a["heads"]), kv_heads=int(a["kv_heads"]), dim=int(a["dim"]), vdim=int(a["vdim"]),
+                conv=int(a["conv"]), window=int(a["mask"]["size"]), keep_first=int(a["mask"]["keep_first"]),
+                rot=_rotary(a["rot"], "pairs"), scale=float(a["scale"]), softcap=float(a["softcap"]))
+            if left.heads % left.kv_heads or left.conv < 1 or left.window < 1 or left.rot.dims > left.dim:
+                raise ValueError(f"layer {i}: heads must be a multiple of kv_heads, conv and window at least 1, "
+                                 "rotary dims within the head")
+            right = GatedRecurrenceSpec(int(r["heads"]), int(r["dim"]), int(r["vdim"]))
+            mixer = ParallelMixerSpec(left, right, float(m["left_scale"]), float(m["right_scale"]))
+        else:
+            raise ValueError(f"layer {i}: unknown mixer type {kind!r}")
+        f = entry.get("mlp")
+        mlp = None
+        if f is not None:
+            if f["kind"] != "dense":
+                raise ValueError(f"layer {i}: unknown feed-forward kind {f['kind']!r}")
+            mlp = FeedForwardSpec(kind="dense", ff=int(f["ff"]), act="xielu")
+        out.append(LayerSpec(kind, mixer, mlp))
+    return tuple(out)
+
+
+def revelix_config(name: str, vocab: int, width: int, layers: list[dict], logit_scale: float = 1.0,
+                   norm_eps: float = 1e-6, max_position_embeddings: int = 32768) -> "ModelConfig":
+    specs = revelix_layers(layers)
+    heads = [s.mixer.left.heads if s.type == "parallel" else s.mixer.heads for s in specs]
+    dims = [s.mixer.left.dim if s.type == "parallel" else s.mixer.dim for s in specs]
+    return ModelConfig(
+        name=name, architecture="revelix", vocab_size=int(vocab), hidden_size=int(width),
+        intermediate_size=max([s.mlp.ff for s in specs if s.mlp] + [0]), num_layers=len(specs),
+        num_heads=max(heads), num_kv_heads=max([s.mixer.left.kv_heads for s in specs if s.type == "parallel"] + [1]),
+        head_dim=max(dims), norm_eps=float(norm_eps), max_position_embeddings=max_position_embeddings,
+        tie_word_embeddings=True, logit_scale=float(logit_scale), layer_specs=specs,
+        bos_token_id=0, eos_token_id=-1)  # the design names no special tokens
 
 
 def zururax_layers(layers: list[dict]) -> tuple:
@@ -119,7 +284,7 @@ def zururax_config(name: str, vocab: int, width: int, layers: list[dict], embedd
 @dataclass
 class ModelConfig:
     name: str = "tiny-llama"
-    architecture: str = "llama"  # llama | mixtral | opt | gpt2 | zururax
+    architecture: str = "llama"  # llama | mixtral | opt | gpt2 | zururax | revelix
     vocab_size: int = 512
     hidden_size: int = 256
     intermediate_size: int = 512
@@ -145,6 +310,7 @@ class ModelConfig:
     # designs whose layers differ from one another list them (Zururax); empty = num_layers equal layers
     layer_specs: tuple = ()
     embedding_scale: float = 1.0
+    logit_scale: float = 1.0   # logits = head(x) * logit_scale
 
     @property
     def q_size(self) -> int:
@@ -161,9 +327,15 @@ class ModelConfig:
             gemm = pair = 0.0
             for s in self.layer_specs:
                 m, f = s.mixer, s.mlp
-                gemm += h * (m.q_rank + m.heads) + m.q_rank * m.heads * (m.dim + m.rot_dim) + m.heads * m.vdim * h
-                gemm += m.heads * m.kv_rank * (m.dim + m.vdim) + (h * m.entry if m.kv_from is None else 0)
-                pair += m.heads * (m.entry + m.kv_rank)
+                gemm += m.weight_count(h)
+                if isinstance(m, LatentMixerSpec):
+                    pair += m.heads * (m.entry + m.kv_rank)
+                else:  # recurrences cost per token, a windowed softmax at most its window per token
+                    for part in (getattr(m, "left", None), getattr(m, "right", None), m):
+                        if hasattr(part, "token_flops"):
+                            gemm += part.token_flops() / 2.0
+                        if isinstance(part, WindowAttentionSpec):
+                            gemm += part.heads * (part.dim + part.kv_heads * part.vdim) * (part.window + part.keep_first)
                 if f is not None:
                     gemm += 2 * h * f.ff if f.kind == "dense" else 3 * h * (f.top * f.ff + f.shared_ff) + h * f.experts
             return 2.0 * gemm, 2.0 * pair
@@ -174,11 +346,10 @@ class ModelConfig:
     def num_params(self) -> int:
         h, i, l_ = self.hidden_size, self.intermediate_size, self.num_layers
         if self.layer_specs:
-            n = 2 * self.vocab_size * h
+            n = self.vocab_size * h * (1 if self.tie_word_embeddings else 2)
             for s in self.layer_specs:
                 m, f = s.mixer, s.mlp
-                n += h * (m.q_rank + m.heads) + m.q_rank * m.heads * (m.dim + m.rot_dim) + m.heads * m.vdim * h
-                n += m.heads * m.kv_rank * (m.dim + m.vdim) + (h * m.entry if m.kv_from is None else 0)
+                n += m.weight_count(h)
                 if f is not None:
                     n += 2 * h * f.ff if f.kind == "dense" else 3 * h * (f.experts * f.ff + f.shared_ff) + h * f.experts
             return n
@@ -342,6 +513,10 @@ def _from_hf_config(cfg: dict[str, Any], name: str) -> ModelConfig:
         return zururax_config(name, cfg["vocab"], cfg["width"], cfg["layers"],
                               embedding_scale=(cfg.get("embedding") or {}).get("scale", 1.0),
                               norm_eps=(cfg.get("norm") or {}).get("eps", 1e-5),
+                              max_position_embeddings=int(cfg.get("max_positions", 32768)))
+    if str(cfg.get("architecture", "")).lower() == "revelix":
+        return revelix_config(name, cfg["vocab"], cfg["width"], cfg["layers"], logit_scale=cfg.get("logit_scale", 1.0),
+                              norm_eps=(cfg.get("norm") or {}).get("eps", 1e-6),
                               max_position_embeddings=int(cfg.get("max_positions", 32768)))
     arch = (cfg.get("architectures") or [""])[0].lower()
     mt = cfg.get("model_type", "").lower()

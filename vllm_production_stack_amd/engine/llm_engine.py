@@ -16,7 +16,7 @@ import uuid
 
 import torch
 
-from .block_manager import PAGE, BlockManager
+from .block_manager import PAGE, BlockManager, StateSlots
 from .config import EngineConfig, resolve_model
 from .metrics import EngineMetrics
 from .model_runner import ModelRunner
@@ -42,10 +42,15 @@ class LLMEngine:
         self.tokenizer = load_tokenizer(self.ckpt_dir, self.model_cfg.vocab_size, cfg.chat_template)
         self.connector = None
         # transfers publish pages through the prefix cache, so a P/D replica always reuses in HBM
-        self.bm = BlockManager(self.runner.num_pages, cfg.enable_prefix_caching or cfg.kv_offload.enabled,
-                               reuse_in_hbm=cfg.enable_prefix_caching or cfg.kv_transfer is not None)
+        # a sequence of a stateful model is its pages AND its state slot: pages found by their hashes do
+        # not bring the state back, so nothing is reused across requests
+        stateful = self.runner.stateful
+        self.bm = BlockManager(self.runner.num_pages,
+                               (cfg.enable_prefix_caching or cfg.kv_offload.enabled) and not stateful,
+                               reuse_in_hbm=(cfg.enable_prefix_caching or cfg.kv_transfer is not None) and not stateful)
         self.scheduler = Scheduler(self.bm, cfg.max_num_seqs, cfg.max_num_batched_tokens,
-                                   self.max_model_len, cfg.enable_chunked_prefill)
+                                   self.max_model_len, cfg.enable_chunked_prefill,
+                                   state_slots=StateSlots(cfg.max_num_seqs) if stateful else None)
         if self.device.type == "cuda" and cfg.prefill_step_ms > 0:
             gemm_f, attn_f = self.model_cfg.prefill_flops()
             tp = max(1, cfg.tensor_parallel_size)

@@ -82,6 +82,10 @@ class ModelRunner:
         self._pool_dev_ptr = 0       # an allocation of our own behind the pool (exported to peers), or 0
         self.pool_ipc_handle = None  # hex hipIpc handle of that allocation
         self.pool = self._alloc_pool()
+        # models whose mixers carry state from token to token: one fp32 slot per running sequence
+        self.stateful = hasattr(self.model, "state_shape")
+        self.state_pool = None
+        self._alloc_state()
         self.sampler = Sampler(device, cfg.seed)
         # graphs need the HIP attention kernels (the generic path reads lengths on the host)
         self.use_graphs = (device.type == "cuda" and not cfg.enforce_eager
@@ -182,6 +186,15 @@ class ModelRunner:
             except Exception as e:
                 log.warning("KV pool could not be exported to prefill peers (%s): pushes land in a window", e)
         return torch.zeros(shape, dtype=self.dtype, device=self.device)
+
+    def _alloc_state(self) -> None:
+        """The per-sequence state pool [max_num_seqs, *model.state_shape()], fp32.  Never cleared: a chunk
+        that starts at position 0 starts from zero state inside the kernels."""
+        if not self.stateful:
+            return
+        self.state_pool = torch.zeros((self.cfg.max_num_seqs, *self.model.state_shape()), dtype=torch.float32,
+                                      device=self.device)
+        self.model.bind_state(self.state_pool)
 
     def _alloc_exported_pool(self) -> torch.Tensor:
         import ctypes
@@ -309,6 +322,8 @@ class ModelRunner:
             plan["pre_pages"] = [s.req.pages for s in prefills]
             plan["q_lens"] = [s.n for s in prefills]
             plan["pre_ctx"] = [s.start + s.n for s in prefills]
+        if self.stateful:
+            plan["state_slots"] = [s.req.state_slot for s in decodes + prefills]
         if self.model.lora is not None:
             lslots = [s.req.lora_slot for s in decodes]
             for s in prefills:
@@ -358,6 +373,8 @@ class ModelRunner:
                 meta.pre_tile_rows = rows
                 meta.pre_tile_seq = self._to_dev(ts, torch.int32)
                 meta.pre_tile_q0 = self._to_dev(tq, torch.int32)
+        if hasattr(self.model, "plan_batch"):  # the sequences of the step and their state slots
+            self.model.plan_batch(meta, plan, self._to_dev)
         rows = plan["logits_rows"]
         meta.logits_rows = self._to_dev(rows, torch.int64) if rows else None
         if plan.get("lora_slots") is not None:
@@ -522,7 +539,10 @@ class ModelRunner:
                 t.untyped_storage().resize_(0)
             except Exception:  # storage that cannot be resized (shared with another process)
                 pass
+        if self.state_pool is not None:
+            self.state_pool.untyped_storage().resize_(0)
         self.pool = None
+        self.state_pool = None
         self.model = None
         self.sampler = None
         gc.collect()
@@ -546,10 +566,11 @@ class ModelRunner:
         # step touches it).  The block-table twin keeps what it holds per row between steps:
         # a row is rewritten only when another request moves into it or its page list grows.
         d64 = torch.zeros((2, bsz), dtype=torch.int64, device=dev)
-        d32 = torch.zeros((2, bsz), dtype=torch.int32, device=dev)
+        d32 = torch.zeros((3, bsz), dtype=torch.int32, device=dev)  # positions | context lengths | state slots
         d64[1].fill_(-1)
+        d32[2].fill_(-1)
         h64 = torch.zeros((2, bsz), dtype=torch.int64)
-        h32 = torch.zeros((2, bsz), dtype=torch.int32)
+        h32 = torch.zeros((3, bsz), dtype=torch.int32)
         hbt = torch.zeros((bsz, mp), dtype=torch.int32)
         if self._pin:
             h64, h32, hbt = h64.pin_memory(), h32.pin_memory(), hbt.pin_memory()
@@ -569,6 +590,8 @@ class ModelRunner:
                          dec_block_tables=st["bt"], dec_ctx_lens=st["ctx"], dec_num_splits=splits,
                          dec_ws_o=ws_o, dec_ws_ml=ws_ml, logits_rows=None,
                          lora_slots=st["lora"] if with_lora else None)
+        if self.stateful:
+            self.model.plan_decode_graph(meta, bsz, d32[2])
 
         def run():
             hidden = self.model.forward(st["ids"], self.pool, meta)
@@ -627,6 +650,8 @@ class ModelRunner:
         for i in range(n, bsz):  # rows past the batch hold no request (ctx 0: nothing is read)
             row_pages[i] = None
         plan = {"bsz": bsz, "ids": ids, "pos": pos, "slots": slots, "ctx": ctx, "bt": bt}
+        if self.stateful:
+            plan["state"] = [s.req.state_slot for s in decodes] + [-1] * (bsz - n)
         if with_lora:
             plan["lora"] = [s.req.lora_slot for s in decodes] + [-1] * (bsz - n)
         if self.distributed:
@@ -918,6 +943,7 @@ class ModelRunner:
             nbt[row, lo:lo + len(pages)] = pages
         n64, n32 = st["n64"], st["n32"]
         n64[0], n64[1], n32[0], n32[1] = plan["ids"], plan["slots"], plan["pos"], plan["ctx"]
+        n32[2] = plan.get("state", -1)
         st["d64"].copy_(st["h64"], non_blocking=True)
         st["d32"].copy_(st["h32"], non_blocking=True)
         if plan["bt"]:
@@ -981,6 +1007,10 @@ class ModelRunner:
         for fn in self.pool_listeners:  # nobody may keep a view of memory that is about to go
             fn(self.pool)
         self._free_exported_pool()  # peers re-map the new allocation (new handle) after the wake-up
+        if self.stateful:  # no sequence is running: nothing in the slots is needed again
+            freed += self.state_pool.numel() * 4
+            self.state_pool = None
+            self.model.bind_state(None)
         if self.device.type == "cuda":
             torch.cuda.empty_cache()
         self.sleeping = True
@@ -1006,6 +1036,7 @@ class ModelRunner:
             self._pack_decode_weights()
         self._sleep_stash = []
         self.pool = self._alloc_pool()
+        self._alloc_state()
         for fn in self.pool_listeners:  # whoever keeps the pool tensor (KV tiers) takes the new one
             fn(self.pool)
         self.sleeping = False

@@ -49,6 +49,7 @@ class Request:
     output_ids: list[int] = field(default_factory=list)
     num_computed: int = 0  # tokens whose KV is resident in this request's pages
     pages: list[int] = field(default_factory=list)
+    state_slot: int = -1  # slot of the per-sequence state pool (stateful models), -1 = none
     hashes: list[int] = field(default_factory=list)  # chain hash per full page (prompt+output)
     num_registered: int = 0  # pages already published to the prefix cache
     num_cached_tokens: int = 0  # prefix tokens served from HBM cache at admission

@@ -17,7 +17,7 @@ import time
 from collections import deque
 from dataclasses import dataclass, field
 
-from .block_manager import PAGE, BlockManager, chain_hashes
+from .block_manager import PAGE, BlockManager, StateSlots, chain_hashes
 from .request import Request, RequestState
 
 
@@ -48,8 +48,10 @@ class SchedulerOutput:
 
 class Scheduler:
     def __init__(self, block_manager: BlockManager, max_num_seqs: int, max_num_batched_tokens: int,
-                 max_model_len: int, enable_chunked_prefill: bool = True, connector=None):
+                 max_model_len: int, enable_chunked_prefill: bool = True, connector=None,
+                 state_slots: StateSlots | None = None):
         self.bm = block_manager
+        self.state_slots = state_slots  # stateful models: a running sequence holds one
         self.max_num_seqs = max_num_seqs
         self.max_model_len = max_model_len
         self.enable_chunked_prefill = enable_chunked_prefill
@@ -110,6 +112,16 @@ class Scheduler:
         req.pages = []
         req.num_computed = 0
         req.num_registered = 0
+        self._drop_state(req)
+
+    def _take_state(self, req: Request) -> None:
+        if self.state_slots is not None and req.state_slot < 0:
+            req.state_slot = self.state_slots.take()
+
+    def _drop_state(self, req: Request) -> None:
+        if self.state_slots is not None and req.state_slot >= 0:
+            self.state_slots.give_back(req.state_slot)
+        req.state_slot = -1
 
     def _ensure_pages(self, req: Request, upto_tokens: int) -> bool:
         need = (upto_tokens + PAGE - 1) // PAGE - len(req.pages)
@@ -250,6 +262,7 @@ class Scheduler:
                 break
             self.waiting.popleft()
             req.state = RequestState.RUNNING
+            self._take_state(req)
             if req.pending_stats is not None:
                 self.bm.queries += req.pending_stats[0]
                 self.bm.hits += req.pending_stats[1]
@@ -275,6 +288,7 @@ class Scheduler:
                 self.waiting.remove(req)
             req.state = RequestState.RUNNING
             self.running.append(req)
+            self._take_state(req)
         if req.num_computed != req.num_tokens:
             raise RuntimeError("a dictated chunk must start where the request's cache ends")
         start, n = req.num_computed, len(tokens)
@@ -318,3 +332,4 @@ class Scheduler:
         if req.pages:
             self.bm.free(req.pages)
             req.pages = []
+        self._drop_state(req)

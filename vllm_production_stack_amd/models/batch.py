@@ -47,3 +47,8 @@ class BatchMeta:
     logits_rows: torch.Tensor | None = None  # int64 [num_out]
     # per-row LoRA slot (-1 = base model), only when adapters are active
     lora_slots: torch.Tensor | None = None
+    # models whose sequences carry state (``model.plan_batch``): every sequence of the step, decode rows
+    # first (one row each), then the prefill chunks
+    seq_cu: torch.Tensor | None = None      # int32 [S + 1]: first row of every sequence
+    seq_state: torch.Tensor | None = None   # int32 [S]: the sequence's state slot, -1 = rows of no sequence
+    row_seq: torch.Tensor | None = None     # int32 [T]: the row's sequence (None: row i is sequence i)

@@ -17,6 +17,7 @@ from ..engine.config import ModelConfig
 from ..parallel.state import get_tp
 from .opt import OPTModel
 from .transformer import LayerWeights, TransformerModel
+from .revelix import RevelixModel
 from .zururax import ZururaxModel
 
 
@@ -27,6 +28,8 @@ def build_model(cfg: ModelConfig, dtype: torch.dtype, device: torch.device, max_
         model = OPTModel(cfg, dtype, device, max_model_len)
     elif cfg.architecture == "zururax":
         model = ZururaxModel(cfg, dtype, device, max_model_len)
+    elif cfg.architecture == "revelix":
+        model = RevelixModel(cfg, dtype, device, max_model_len)
     else:
         model = TransformerModel(cfg, dtype, device, max_model_len, expert_parallel=expert_parallel)
     has_weights = ckpt_dir is not None and any(Path(ckpt_dir).glob("*.safetensors"))
@@ -58,6 +61,8 @@ def load_hf_weights(model, ckpt_dir: Path) -> None:
         (_load_gpt2 if model.cfg.architecture == "gpt2" else _load_opt)(model, ckpt_dir)
     elif isinstance(model, ZururaxModel):
         _load_zururax(model, ckpt_dir)
+    elif isinstance(model, RevelixModel):
+        _load_revelix(model, ckpt_dir)
     else:
         _load_llama(model, ckpt_dir)
 
@@ -326,5 +331,132 @@ def _load_zururax(model: ZururaxModel, ckpt_dir: Path) -> None:
                 want |= {f"l{i}.mlp.e{e}.{k}" for e in range(f.experts) for k in ("gate", "up", "down")}
                 if f.shared_ff:
                     want |= {f"l{i}.mlp.shared.{k}" for k in ("gate", "up", "down", "sg")}
+    if want - seen:
+        raise ValueError(f"checkpoint lacks {sorted(want - seen)[:8]}")
+
+
+def _load_revelix(model: RevelixModel, ckpt_dir: Path) -> None:
+    """Revelix checkpoints: ``embed``; per layer ``l<i>.norm1|norm2`` with ``.b`` and ``.alpha``;
+    ``l<i>.mix.{q, k, v, g, o}`` (retention) or ``l<i>.mix.left.{q, k, v (each with .b and .conv), talk, sink, o}``
+    and ``l<i>.mix.right.{q, f, f.b, lower, v, norm, o}`` (parallel); ``l<i>.mlp.{up, down, act}``;
+    ``final.norm`` (+ ``.b``, ``.alpha``).  Linear weights are [out, in]; the input projections of a
+    mixer are fused row-wise here.  Every tensor the model holds must be found, and every tensor of the
+    file must have a place."""
+    from ..engine.config import ParallelMixerSpec
+
+    pat = re.compile(r"l(\d+)\.(.+)")
+    seen: set[str] = set()
+
+    def put(dst: torch.Tensor, src: torch.Tensor, what: str) -> None:
+        if tuple(dst.shape) != tuple(src.shape):
+            raise ValueError(f"{what}: checkpoint shape {tuple(src.shape)}, model expects {tuple(dst.shape)}")
+        dst.copy_(src.to(dst.dtype))
+
+    def put_norm(norm: list, which: str, src: torch.Tensor, what: str) -> bool:
+        i = {"": 0, ".b": 1, ".alpha": 2}.get(which)
+        if i is None:
+            return False
+        put(norm[i], src.reshape(norm[i].shape) if i == 2 and src.numel() == 1 else src, what)
+        return True
+
+    for name, t in _iter_safetensors(ckpt_dir):
+        seen.add(name)
+        if name == "embed":
+            put(model.embed, t, name)
+            continue
+        if name.startswith("final.norm"):
+            if not put_norm(model.norm, name[len("final.norm"):], t, name):
+                raise ValueError(f"unexpected tensor {name!r}")
+            continue
+        mt = pat.match(name)
+        if not mt or int(mt.group(1)) >= len(model.layers):
+            raise ValueError(f"unexpected tensor {name!r}")
+        lw = model.layers[int(mt.group(1))]
+        sub = mt.group(2)
+        m, f = lw.spec.mixer, lw.spec.mlp
+        ok = False
+        if sub.startswith("norm1"):
+            ok = put_norm(lw.norm1, sub[5:], t, name)
+        elif sub.startswith("norm2") and f is not None:
+            ok = put_norm(lw.norm2, sub[5:], t, name)
+        elif sub.startswith("mlp.") and f is not None:
+            ok = True
+            if sub == "mlp.up":
+                put(lw.w_up, t, name)
+            elif sub == "mlp.down":
+                put(lw.w_down, t, name)
+            elif sub == "mlp.act":
+                p = t.double()
+                if p.numel() != 2:
+                    raise ValueError(f"{name}: two numbers expected")
+                sp = torch.nn.functional.softplus(p)
+                lw.act.copy_(torch.stack([sp[0], 0.5 + sp[1]]).float())
+            else:
+                ok = False
+        elif not isinstance(m, ParallelMixerSpec):
+            hd, hv = m.heads * m.dim, m.heads * m.vdim
+            rows = {"mix.q": (0, hd), "mix.k": (hd, 2 * hd), "mix.v": (2 * hd, 2 * hd + hv),
+                    "mix.g": (2 * hd + hv, 2 * hd + 2 * hv)}
+            if sub in rows:
+                a, b = rows[sub]
+                put(lw.w_in[a:b], t, name)
+                ok = True
+            elif sub == "mix.o":
+                put(lw.w_o, t, name)
+                ok = True
+        else:
+            a, r = m.left, m.right
+            nq, nk, nv = a.heads * a.dim, a.kv_heads * a.dim, a.kv_heads * a.vdim
+            c0, rd = a.channels, r.heads * r.dim
+            left = {"q": (0, nq), "k": (nq, nq + nk), "v": (nq + nk, nq + nk + nv)}
+            right = {"q": (c0, c0 + rd), "f": (c0 + rd, c0 + 2 * rd), "v": (c0 + 2 * rd, c0 + 2 * rd + r.heads * r.vdim)}
+            ok = True
+            parts = sub.split(".")
+            if sub.startswith("mix.left.") and len(parts) >= 3 and parts[2] in left:
+                lo, hi = left[parts[2]]
+                rest = ".".join(parts[3:])
+                if rest == "":
+                    put(lw.w_in[lo:hi], t, name)
+                elif rest == "b":
+                    put(lw.b_in[lo:hi], t, name)
+                elif rest == "conv":
+                    put(lw.conv_w[lo:hi], t, name)
+                else:
+                    ok = False
+            elif sub == "mix.left.talk":
+                put(lw.talk, t, name)
+            elif sub == "mix.left.sink":
+                put(lw.sink, t, name)
+            elif sub == "mix.left.o":
+                put(lw.w_o, t, name)
+            elif sub.startswith("mix.right.") and len(parts) == 3 and parts[2] in right:
+                lo, hi = right[parts[2]]
+                put(lw.w_in[lo:hi], t, name)
+            elif sub == "mix.right.f.b":
+                put(lw.gate_bias, t, name)
+            elif sub == "mix.right.lower":
+                put(lw.gate_lower, t, name)
+            elif sub == "mix.right.norm":
+                put(lw.r_norm, t, name)
+            elif sub == "mix.right.o":
+                put(lw.wr_o, t, name)
+            else:
+                ok = False
+        if not ok:
+            raise ValueError(f"unexpected tensor {name!r}")
+    want = {"embed"} | {"final.norm" + x for x in ("", ".b", ".alpha")}
+    for i, lw in enumerate(model.layers):
+        m, f = lw.spec.mixer, lw.spec.mlp
+        want |= {f"l{i}.norm1{x}" for x in ("", ".b", ".alpha")}
+        if isinstance(m, ParallelMixerSpec):
+            for k in ("q", "k", "v"):
+                want |= {f"l{i}.mix.left.{k}", f"l{i}.mix.left.{k}.b", f"l{i}.mix.left.{k}.conv"}
+            want |= {f"l{i}.mix.left.{k}" for k in ("talk", "sink", "o")}
+            want |= {f"l{i}.mix.right.{k}" for k in ("q", "f", "f.b", "lower", "v", "norm", "o")}
+        else:
+            want |= {f"l{i}.mix.{k}" for k in ("q", "k", "v", "g", "o")}
+        if f is not None:
+            want |= {f"l{i}.norm2{x}" for x in ("", ".b", ".alpha")}
+            want |= {f"l{i}.mlp.{k}" for k in ("up", "down", "act")}
     if want - seen:
         raise ValueError(f"checkpoint lacks {sorted(want - seen)[:8]}")

@@ -41,6 +41,8 @@ def _kernels():
             "vpsa_latent_attention", "vpsa_sigmoid_gate", "vpsa_relu_sq", "vpsa_glu_clamp", "vpsa_group_topk",
             "vpsa_gather_rows", "vpsa_moe_finish", "vpsa_latent_mfma_supported", "vpsa_latent_attention_mfma",
             "vpsa_moe_mfma_act",
+            "vpsa_add_dyt", "vpsa_recurrent_scan", "vpsa_head_rms", "vpsa_short_conv_qkv", "vpsa_window_attention",
+            "vpsa_mix_heads", "vpsa_xielu",
         ):
             getattr(lib, name).restype = c_int
         lib.vpsa_prefill_split_record_bytes.restype = c_long
@@ -1325,3 +1327,7 @@ def lora_expand(h, bs, slots, y, r_pad):
 from .latent import (add_rms_norm, build_latent_tiles, embed_scale, gate_up_glu_clamp, gather_rows, glu_clamp,  # noqa: E402,F401
                      group_topk, latent_attention, moe_glu_grouped, moe_glu_grouped_supported, up_relu_sq,
                      latent_kv_write, latent_mfma_supported, latent_tile_kernel_takes, moe_finish, relu_sq, rms_norm_rows, rope_pairs, sigmoid_gate)
+
+# --------------------------------------------------------------------------- recurrent mixers, windowed attention, Dynamic Tanh
+from .seqmix import (add_dyt_norm, head_rms_norm, mix_heads, recurrent_scan, short_conv_qkv, up_xielu,  # noqa: E402,F401
+                     window_attention, window_cache_elems, xielu)

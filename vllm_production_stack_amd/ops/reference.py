@@ -49,8 +49,25 @@ def build_cos_sin(head_dim: int, max_pos: int, theta: float, scaling: dict | Non
         mid = (1 - smooth) * inv / factor + smooth * inv
         is_mid = (wavelen <= orig / lo) & (wavelen >= orig / hi)
         inv = torch.where(is_mid, mid, scaled)
+    mag = 1.0
+    if scaling and scaling.get("rope_type", scaling.get("type")) == "ramp":
+        # frequencies divided by ``factor`` behind a linear ramp over the pair index, between the pairs
+        # that make ``fast`` and ``slow`` turns over ``original`` positions; cos and sin grow by
+        # 0.1 ln(factor) + 1
+        import math
+
+        factor, orig = float(scaling["factor"]), float(scaling["original"])
+
+        def pair_of(turns):
+            return head_dim * math.log(orig / (2 * math.pi * turns)) / (2 * math.log(theta))
+
+        lo = max(math.floor(pair_of(float(scaling["fast"]))), 0)
+        hi = min(math.ceil(pair_of(float(scaling["slow"]))), head_dim - 1)
+        ramp = ((torch.arange(0, half, dtype=torch.float64) - lo) / max(hi - lo, 0.001)).clamp(0, 1)
+        inv = inv / factor * ramp + inv * (1 - ramp)
+        mag = 0.1 * math.log(factor) + 1.0
     ang = torch.arange(max_pos, dtype=torch.float64)[:, None] * inv[None, :]
-    return torch.cat([ang.cos(), ang.sin()], dim=-1).float().to(device)
+    return (torch.cat([ang.cos(), ang.sin()], dim=-1) * mag).float().to(device)
 
 
 def _kv_views(pool, layer, n_kv, head_dim):
@@ -445,3 +462,153 @@ def moe_finish(residual, y, weights, pos, shared, gate):
     if shared is not None:
         residual.add_(shared.float() * (gate[:, None] if gate is not None else 1.0))
     return residual
+
+
+# --------------------------------------------------------------------------- recurrent mixers, windowed attention, Dynamic Tanh
+def add_dyt_norm(residual, deltas, weight, bias, alpha, out_dtype, want_out=True):
+    for d, scale in deltas:
+        residual.add_(d.float() * scale)
+    if not want_out:
+        return None
+    return (torch.tanh(residual * alpha) * weight + bias).to(out_dtype)
+
+
+def _rotate_rows(x, pos, cos_sin, dims, layout):
+    """x fp32 [T, heads, d]: the first ``dims`` channels of every head turn by the table row of the
+    token's position; pairs (i, i + dims / 2) for layout 0, (2 i, 2 i + 1) for layout 1."""
+    if dims == 0:
+        return x
+    cs = cos_sin[pos.long()]
+    c, s = cs[:, None, :dims // 2], cs[:, None, dims // 2:]
+    out = x.clone()
+    if layout == 0:
+        u, v = x[..., :dims // 2], x[..., dims // 2:dims]
+        out[..., :dims // 2] = u * c - v * s
+        out[..., dims // 2:dims] = v * c + u * s
+    else:
+        u, v = x[..., 0:dims:2], x[..., 1:dims:2]
+        out[..., 0:dims:2] = u * c - v * s
+        out[..., 1:dims:2] = v * c + u * s
+    return out
+
+
+def recurrent_scan(proj, q_col, k_col, v_col, heads, dim, vdim, gated, state, state_off, seq_cu, seq_state, positions,
+                   decay, cos_sin, rot_dims, layout, k_scale, gate_bias, gate_lower):
+    t = proj.shape[0]
+    out = torch.zeros((t, heads, vdim), dtype=torch.float32)
+    q = proj[:, q_col:q_col + heads * dim].float().view(t, heads, dim)
+    k = proj[:, k_col:k_col + heads * dim].float().view(t, heads, dim)
+    v = proj[:, v_col:v_col + heads * vdim].float().view(t, heads, vdim)
+    if gated:
+        q = torch.nn.functional.silu(q)
+        lower = gate_lower.view(1, heads, dim)
+        a = lower + (1 - lower) * torch.sigmoid(k + gate_bias.view(1, heads, dim))
+        k = 1 - a
+    else:
+        q = _rotate_rows(q, positions, cos_sin, rot_dims, layout)
+        k = _rotate_rows(k, positions, cos_sin, rot_dims, layout) * k_scale
+        a = decay.view(1, heads, 1).expand(t, heads, dim)
+    cu, slots = seq_cu.tolist(), seq_state.tolist()
+    for s, slot in enumerate(slots):
+        r0, r1 = cu[s], cu[s + 1]
+        if slot < 0 or r1 <= r0:
+            continue
+        S = state[slot, state_off:state_off + heads * dim * vdim].view(heads, dim, vdim)
+        if int(positions[r0]) == 0:
+            S.zero_()
+        for r in range(r0, r1):
+            S.mul_(a[r].unsqueeze(-1)).add_(k[r].unsqueeze(-1) * v[r].unsqueeze(1))
+            out[r] = torch.einsum("hdv,hd->hv", S, q[r])
+    return out
+
+
+def head_rms_norm(o, eps, weight, gate, out_dtype):
+    t, heads, vdim = o.shape
+    y = o * torch.rsqrt(o.pow(2).mean(-1, keepdim=True) + eps)
+    if weight is not None:
+        y = y * weight
+    y = y.reshape(t, heads * vdim)
+    if gate is not None:
+        y = y * torch.nn.functional.silu(gate.float())
+    return y.to(out_dtype)
+
+
+def window_cache_views(pool, cache_off, kv_heads, dim, vdim):
+    """K [pages, PAGE, kv_heads, dim] and V [pages, PAGE, kv_heads, vdim] of one layer (views of the pool)."""
+    nk, nv = PAGE * kv_heads * dim, PAGE * kv_heads * vdim
+    k = pool[:, cache_off:cache_off + nk].view(pool.shape[0], PAGE, kv_heads, dim)
+    v = pool[:, cache_off + nk:cache_off + nk + nv].view(pool.shape[0], PAGE, kv_heads, vdim)
+    return k, v
+
+
+def short_conv_qkv(proj, conv_w, heads, kv_heads, dim, vdim, state, state_off, seq_cu, seq_state, positions, slots,
+                   cos_sin, rot_dims, layout, pool, cache_off):
+    t = proj.shape[0]
+    taps = conv_w.shape[1]
+    chans = heads * dim + kv_heads * (dim + vdim)
+    u = proj[:, :chans].float()
+    y = torch.zeros((t, chans), dtype=torch.float32)
+    cu, st = seq_cu.tolist(), seq_state.tolist()
+    for s, slot in enumerate(st):
+        r0, r1 = cu[s], cu[s + 1]
+        if slot < 0 or r1 <= r0:
+            continue
+        tail = state[slot, state_off:state_off + (taps - 1) * chans].view(taps - 1, chans)
+        if int(positions[r0]) == 0:
+            tail.zero_()
+        ext = torch.cat([tail, u[r0:r1]], dim=0)  # the rows before the chunk, then the chunk
+        n = r1 - r0
+        for j in range(taps):
+            y[r0:r1] += conv_w[:, j] * ext[j:j + n]
+        if taps > 1:
+            tail.copy_(ext[n:n + taps - 1].clone())
+    y = y.to(proj.dtype).float()
+    nq, nk = heads * dim, kv_heads * dim
+    q = _rotate_rows(y[:, :nq].reshape(t, heads, dim), positions, cos_sin, rot_dims, layout).to(proj.dtype)
+    k = _rotate_rows(y[:, nq:nq + nk].reshape(t, kv_heads, dim), positions, cos_sin, rot_dims, layout).to(pool.dtype)
+    v = y[:, nq + nk:].reshape(t, kv_heads, vdim).to(pool.dtype)
+    kc, vc = window_cache_views(pool, cache_off, kv_heads, dim, vdim)
+    ok = slots >= 0
+    pg, off = (slots[ok] // PAGE).long(), (slots[ok] % PAGE).long()
+    kc[pg, off] = k[ok]
+    vc[pg, off] = v[ok]
+    return q
+
+
+def window_attention(q, pool, cache_off, kv_heads, vdim, block_tables, row_seq, positions, window, keep_first, scale,
+                     softcap, sink, out):
+    t, heads, dim = q.shape
+    kc, vc = window_cache_views(pool, cache_off, kv_heads, dim, vdim)
+    rep = heads // kv_heads
+    for r in range(t):
+        s = r if row_seq is None else int(row_seq[r])
+        p = int(positions[r])
+        lo = max(0, p - window + 1)
+        keys = list(range(min(keep_first, lo))) + list(range(lo, p + 1))
+        idx = torch.tensor(keys)
+        pages = block_tables[s].long()[idx // PAGE]
+        kk = kc[pages, idx % PAGE].float()       # [keys, kv_heads, dim]
+        vv = vc[pages, idx % PAGE].float()       # [keys, kv_heads, vdim]
+        sc = torch.einsum("hd,khd->hk", q[r].float(), kk.repeat_interleave(rep, dim=1)) * scale
+        sc = softcap * torch.tanh(sc / softcap)
+        mx = torch.maximum(sc.max(-1).values, sink)
+        e = torch.exp(sc - mx[:, None])
+        w = e / (e.sum(-1) + torch.exp(sink - mx))[:, None]
+        out[r] = torch.einsum("hk,kgv->hgv", w, vv)
+    return out
+
+
+def mix_heads(u, talk, out_dtype):
+    t, heads, kv_heads, vdim = u.shape
+    rep = heads // kv_heads
+    own = torch.arange(heads) // rep
+    # out[t, h] = sum_g talk[h, g] u[t, g, kv(h)]
+    sel = u[:, :, own, :]                          # [t, g, h, vdim]
+    return torch.einsum("hg,tghv->thv", talk, sel).reshape(t, heads * vdim).to(out_dtype)
+
+
+def xielu(x, act):
+    z = x.float()
+    pos = act[0] * z * z + 0.5 * z
+    neg = act[1] * (torch.expm1(z) - z) + 0.5 * z
+    return torch.where(z > 0, pos, neg).to(x.dtype)

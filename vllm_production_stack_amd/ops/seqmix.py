@@ -1,0 +1,243 @@
+"""Ops of sequence mixers that carry state from token to token (``csrc/kernels/seqmix.hip``):
+linear-attention recurrences, a short convolution in front of a windowed softmax attention with
+kept first tokens, a sink and post-softmax head mixing, the Dynamic Tanh norm on the fp32 residual
+stream and the xIELU activation.  Device tensors run the HIP kernels in bf16 or fp32 activations;
+CPU tensors run the PyTorch definitions of ``reference.py``.
+
+Two stores, both owned by the engine's runner:
+
+- the paged pool ``[pages, page_elems]`` (activation dtype): a layer with windowed attention keeps, per
+  page and ``cache_off`` elements into it, ``K [PAGE, kv_heads * dim]`` then ``V [PAGE, kv_heads * vdim]``;
+- the state pool ``[slots, state_elems]`` (fp32): a sequence's slot holds, per layer and ``state_off``
+  elements into it, a recurrence's ``[heads, dim, vdim]`` matrix or the ``conv - 1`` projected rows
+  a convolution still needs.  A chunk that starts at position 0 starts from zeros, whatever the slot
+  held before.
+
+A batch is described by ``seq_cu`` (int32 [S + 1]: first row of every sequence, decode rows are
+sequences of one row), ``seq_state`` (int32 [S]: the sequence's slot, -1 = rows of no sequence) and,
+for row-wise kernels, ``row_seq`` (int32 [T], None = row i is sequence i).
+"""
+
+from __future__ import annotations
+
+from ctypes import c_float, c_int, c_long, c_void_p
+
+import torch
+
+from . import reference
+from .reference import PAGE
+
+_DT = {torch.bfloat16: 0, torch.float32: 1}
+
+
+def _ops():
+    from .. import ops
+
+    return ops
+
+
+def _dt(*ts) -> int:
+    d = None
+    for t in ts:
+        if t is None:
+            continue
+        if not t.is_cuda or t.dtype not in _DT:
+            raise TypeError("sequence-mixer kernels take bf16 or fp32 device tensors")
+        if d is not None and _DT[t.dtype] != d:
+            raise TypeError("sequence-mixer kernels: mixed activation dtypes")
+        d = _DT[t.dtype]
+    return d
+
+
+def _f32(*ts):
+    for t in ts:
+        if t is not None and (t.dtype != torch.float32 or not t.is_contiguous()):
+            raise TypeError("expected a contiguous fp32 tensor")
+
+
+def _i32(*ts):
+    for t in ts:
+        if t is not None and (t.dtype != torch.int32 or not t.is_contiguous()):
+            raise TypeError("expected a contiguous int32 tensor")
+
+
+def _rows(t) -> bool:
+    return t.dim() == 2 and t.stride(1) == 1
+
+
+def _at(t, offset: int):
+    return c_void_p(t.data_ptr() + offset * t.element_size())
+
+
+def add_dyt_norm(residual, deltas, weight, bias, alpha, out_dtype, want_out: bool = True):
+    """residual (fp32, in place) += sum of scale * delta over ``deltas`` (up to two (tensor, scale)
+    pairs); returns tanh(alpha * residual) * weight + bias in ``out_dtype`` (Dynamic Tanh: no mean, no
+    variance).  ``alpha`` is a one-element fp32 tensor."""
+    if not residual.is_cuda:
+        return reference.add_dyt_norm(residual, deltas, weight, bias, alpha, out_dtype, want_out)
+    o = _ops()
+    _f32(residual, weight, bias, alpha)
+    t, n = residual.shape
+    assert len(deltas) <= 2
+    if not deltas and not want_out:
+        return None
+    ds = list(deltas) + [(None, 0.0)] * (2 - len(deltas))
+    for d, _ in ds:
+        assert d is None or (_rows(d) and d.shape == residual.shape and d.dtype == out_dtype)
+    y = torch.empty((t, n), dtype=out_dtype, device=residual.device) if want_out else None
+    (d1, c1), (d2, c2) = ds
+    o._check(o._kernels().vpsa_add_dyt(o._p(residual), o._p(d1), c_long(d1.stride(0) if d1 is not None else 0),
+                                       c_float(c1), o._p(d2), c_long(d2.stride(0) if d2 is not None else 0), c_float(c2),
+                                       o._p(weight), o._p(bias), o._p(alpha), o._p(y), c_int(t), c_int(n),
+                                       c_int(_DT[out_dtype]), o._stream()), "add_dyt_norm")
+    return y
+
+
+def recurrent_scan(proj, q_col: int, k_col: int, v_col: int, heads: int, dim: int, vdim: int, state, state_off: int,
+                   seq_cu, seq_state, positions, *, decay=None, cos_sin=None, rot_dims: int = 0, layout: int = 0,
+                   k_scale: float = 1.0, gate_bias=None, gate_lower=None):
+    """Per sequence and head, over the sequence's rows in order: S <- a_t (.) S + k_t v_t^T, o_t = S^T q_t
+    with S [dim, vdim] carried in the sequence's state slot.  q, k and v are column ranges of ``proj``
+    [T, cols] (heads side by side).
+
+    ``decay`` (fp32 [heads]): a_t = decay[head] for every row of S; q and k turn by the rotary table
+    ``cos_sin`` over their first ``rot_dims`` channels (``layout`` 0: pairs (i, i + rot_dims / 2), 1: pairs
+    (2 i, 2 i + 1)) and k is multiplied by ``k_scale`` afterwards.
+
+    ``gate_bias`` / ``gate_lower`` (fp32 [heads * dim]) instead: the k columns hold gate logits,
+    a_t = lower + (1 - lower) sigmoid(logit + bias) per row of S, k_t = 1 - a_t, q = silu(q).
+
+    Returns o fp32 [T, heads, vdim]."""
+    gated = decay is None
+    if not proj.is_cuda:
+        return reference.recurrent_scan(proj, q_col, k_col, v_col, heads, dim, vdim, gated, state, state_off, seq_cu,
+                                        seq_state, positions, decay, cos_sin, rot_dims, layout, k_scale, gate_bias,
+                                        gate_lower)
+    o = _ops()
+    _f32(state, decay, cos_sin, gate_bias, gate_lower)
+    _i32(seq_cu, seq_state, positions)
+    assert _rows(proj) and max(q_col, k_col) + heads * dim <= proj.shape[1] and v_col + heads * vdim <= proj.shape[1]
+    assert state_off + heads * dim * vdim <= state.shape[1] and seq_cu.numel() == seq_state.numel() + 1
+    assert (gate_bias is not None and gate_lower is not None) if gated else (rot_dims == 0 or cos_sin.shape[1] == rot_dims)
+    assert rot_dims <= dim and rot_dims % 2 == 0
+    out = torch.empty((proj.shape[0], heads, vdim), dtype=torch.float32, device=proj.device)
+    o._check(o._kernels().vpsa_recurrent_scan(
+        o._p(proj), c_long(proj.stride(0)), c_int(q_col), c_int(k_col), c_int(v_col), c_int(heads), c_int(dim),
+        c_int(vdim), _at(state, state_off), c_long(state.stride(0)), o._p(seq_cu), o._p(seq_state),
+        c_int(seq_state.numel()), o._p(positions), o._p(decay), o._p(cos_sin), c_int(rot_dims), c_int(layout),
+        c_float(k_scale), o._p(gate_bias), o._p(gate_lower), o._p(out), c_int(1 if gated else 0), c_int(_dt(proj)),
+        o._stream()), "recurrent_scan")
+    return out
+
+
+def head_rms_norm(o_heads, eps: float, out_dtype, weight=None, gate=None):
+    """o fp32 [T, heads, vdim] -> [T, heads * vdim] in ``out_dtype``: every head divided by its root mean
+    square (eps inside the root), times ``weight`` (fp32 [vdim], shared by the heads) and times
+    silu(``gate``) (a [T, heads * vdim] view of a wider projection) where given."""
+    if not o_heads.is_cuda:
+        return reference.head_rms_norm(o_heads, eps, weight, gate, out_dtype)
+    o = _ops()
+    _f32(o_heads, weight)
+    t, heads, vdim = o_heads.shape
+    assert gate is None or (_rows(gate) and gate.shape == (t, heads * vdim) and gate.dtype == out_dtype)
+    y = torch.empty((t, heads * vdim), dtype=out_dtype, device=o_heads.device)
+    o._check(o._kernels().vpsa_head_rms(o._p(o_heads), o._p(weight), o._p(gate),
+                                        c_long(gate.stride(0) if gate is not None else 0), o._p(y), c_int(t),
+                                        c_int(heads), c_int(vdim), c_float(eps), c_int(_DT[out_dtype]), o._stream()),
+             "head_rms_norm")
+    return y
+
+
+def window_cache_elems(kv_heads: int, dim: int, vdim: int) -> int:
+    """Elements a windowed-attention layer keeps per page."""
+    return PAGE * kv_heads * (dim + vdim)
+
+
+def short_conv_qkv(proj, conv_w, heads: int, kv_heads: int, dim: int, vdim: int, state, state_off: int, row_seq, seq_cu,
+                   seq_state, positions, slots, cos_sin, rot_dims: int, layout: int, pool, cache_off: int):
+    """The fused q | k | v projection rows ``proj`` [T, >= channels] through a causal convolution over
+    time on every channel (``conv_w`` fp32 [channels, taps]: y_t = sum_j w[:, j] u_(t - taps + 1 + j), zeros
+    before position 0; the rows before a chunk come from the sequence's state slot, which afterwards
+    holds the chunk's last taps - 1 rows), then the rotary table on q and k.  k and v go to the paged
+    cache at ``slots`` (< 0: not cached); returns q [T, heads, dim]."""
+    if not proj.is_cuda:
+        return reference.short_conv_qkv(proj, conv_w, heads, kv_heads, dim, vdim, state, state_off, seq_cu, seq_state,
+                                        positions, slots, cos_sin, rot_dims, layout, pool, cache_off)
+    o = _ops()
+    _f32(state, conv_w, cos_sin)
+    _i32(row_seq, seq_cu, seq_state, positions)
+    t = proj.shape[0]
+    chans = heads * dim + kv_heads * (dim + vdim)
+    taps = conv_w.shape[1]
+    assert _rows(proj) and proj.shape[1] >= chans and conv_w.shape[0] == chans and slots.dtype == torch.int64
+    assert state_off + (taps - 1) * chans <= state.shape[1] and (rot_dims == 0 or cos_sin.shape[1] == rot_dims)
+    assert pool.dim() == 2 and pool.stride(1) == 1 and cache_off + window_cache_elems(kv_heads, dim, vdim) <= pool.shape[1]
+    assert row_seq is None or row_seq.numel() == t
+    q = torch.empty((t, heads, dim), dtype=proj.dtype, device=proj.device)
+    o._check(o._kernels().vpsa_short_conv_qkv(
+        o._p(proj), c_long(proj.stride(0)), o._p(conv_w), c_int(taps), c_int(heads), c_int(kv_heads), c_int(dim),
+        c_int(vdim), _at(state, state_off), c_long(state.stride(0)), o._p(row_seq), o._p(seq_cu), o._p(seq_state),
+        c_int(seq_state.numel()), o._p(positions), o._p(slots), o._p(cos_sin), c_int(rot_dims), c_int(layout), o._p(q),
+        _at(pool, cache_off), c_long(pool.stride(0)), c_int(t), c_int(_dt(proj, pool)), o._stream()), "short_conv_qkv")
+    return q
+
+
+def window_attention(q, pool, cache_off: int, kv_heads: int, vdim: int, block_tables, row_seq, positions, window: int,
+                     keep_first: int, scale: float, softcap: float, sink, out=None):
+    """Query rows q [T, heads, dim] over their sequences' cached keys: row i at position p sees key j when
+    j <= p and (p - j < window or j < keep_first).  score = cap * tanh(q . k * scale / cap) (cap 0: none);
+    softmax with ``sink`` [heads] (fp32) in the denominator.  Returns u fp32 [T, heads, kv_heads, vdim]:
+    each head's weights applied to the values of every KV head (``mix_heads`` picks and mixes)."""
+    t, heads, dim = q.shape
+    if out is None:
+        out = torch.empty((t, heads, kv_heads, vdim), dtype=torch.float32, device=q.device)
+    if t == 0:
+        return out
+    if not q.is_cuda:
+        return reference.window_attention(q, pool, cache_off, kv_heads, vdim, block_tables, row_seq, positions, window,
+                                          keep_first, scale, softcap, sink, out)
+    o = _ops()
+    _f32(sink, out)
+    _i32(row_seq, positions)
+    assert q.stride(2) == 1 and q.stride(1) == dim and block_tables.dtype == torch.int32 and block_tables.stride(1) == 1
+    assert heads % kv_heads == 0 and cache_off + window_cache_elems(kv_heads, dim, vdim) <= pool.shape[1]
+    o._check(o._kernels().vpsa_window_attention(
+        o._p(q), c_long(q.stride(0)), _at(pool, cache_off), c_long(pool.stride(0)), o._p(block_tables),
+        c_int(block_tables.stride(0)), o._p(row_seq), o._p(positions), o._p(sink), o._p(out), c_int(t), c_int(heads),
+        c_int(kv_heads), c_int(dim), c_int(vdim), c_int(window), c_int(keep_first), c_float(scale), c_float(softcap),
+        c_int(_dt(q, pool)), o._stream()), "window_attention")
+    return out
+
+
+def mix_heads(u, talk, out_dtype):
+    """u fp32 [T, heads, kv_heads, vdim], talk fp32 [heads, heads] -> [T, heads * vdim]:
+    out[t, h] = sum_g talk[h, g] * u[t, g, kv head of h] (softmax weights mixed across heads, each head
+    keeping its own values)."""
+    if not u.is_cuda:
+        return reference.mix_heads(u, talk, out_dtype)
+    o = _ops()
+    _f32(u, talk)
+    t, heads, kv_heads, vdim = u.shape
+    y = torch.empty((t, heads * vdim), dtype=out_dtype, device=u.device)
+    o._check(o._kernels().vpsa_mix_heads(o._p(u), o._p(talk), o._p(y), c_int(t), c_int(heads), c_int(kv_heads),
+                                         c_int(vdim), c_int(_DT[out_dtype]), o._stream()), "mix_heads")
+    return y
+
+
+def xielu(x, act):
+    """z > 0: act[0] z^2 + z / 2; else act[1] (exp(z) - 1 - z) + z / 2.  ``act`` fp32 [2] on the device
+    (softplus of the first learned number, 1/2 + softplus of the second)."""
+    if not x.is_cuda:
+        return reference.xielu(x, act)
+    o = _ops()
+    _f32(act)
+    assert x.is_contiguous()
+    y = torch.empty_like(x)
+    o._check(o._kernels().vpsa_xielu(o._p(x), o._p(y), c_long(x.numel()), o._p(act), c_int(_dt(x)), o._stream()),
+             "xielu")
+    return y
+
+
+def up_xielu(x, w_up, act):
+    """xielu(x @ W.T)."""
+    return xielu(_ops().linear(x, w_up), act)
