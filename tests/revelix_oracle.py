@@ -77,6 +77,18 @@ def xielu(z, p, q):
     return torch.where(z > 0, pos, neg)
 
 
+def linear_recurrence(q, k, v, a):
+    """q, k, a [T, H, d], v [T, H, vd]: per head S_t = diag(a_t) S_(t-1) + k_t v_t^T from S = 0, o_t = S_t^T q_t."""
+    t, H, d = q.shape
+    o = torch.zeros(t, H, v.shape[-1], dtype=F64)
+    for hd in range(H):
+        S = torch.zeros(d, v.shape[-1], dtype=F64)
+        for i in range(t):
+            S = a[i, hd][:, None] * S + torch.outer(k[i, hd], v[i, hd])
+            o[i, hd] = S.T @ q[i, hd]
+    return o
+
+
 def retention(h, W, m: dict, eps: float):
     """The mixer of a 'retention' layer over one sequence h [T, width]."""
     t = h.shape[0]
@@ -85,14 +97,34 @@ def retention(h, W, m: dict, eps: float):
     q = rotate((h @ W["q"].T).view(t, H, d), pos, m["rot"], "half")
     k = rotate((h @ W["k"].T).view(t, H, d), pos, m["rot"], "half") * d ** -0.5
     v = (h @ W["v"].T).view(t, H, vd)
-    o = torch.zeros(t, H, vd, dtype=F64)
-    for hd in range(H):
-        S = torch.zeros(d, vd, dtype=F64)
-        for i in range(t):
-            S = float(m["decay"][hd]) * S + torch.outer(k[i, hd], v[i, hd])
-            o[i, hd] = S.T @ q[i, hd]
+    decay = torch.tensor(m["decay"], dtype=F64).view(1, H, 1).expand(t, H, d)
+    o = linear_recurrence(q, k, v, decay)
     o = rms_unit(o, eps).reshape(t, H * vd) * torch.nn.functional.silu(h @ W["g"].T)
     return o @ W["o"].T
+
+
+def window_weights(q, k, pos_q, pos_k, heads_per_kv: int, scale, cap, size, keep, sink):
+    """Softmax weights [H, Tq, Tk] of queries at positions pos_q over keys at positions pos_k: capped
+    scores, the window with kept first tokens, the sink in the denominator only."""
+    H = q.shape[1]
+    i, j = pos_q[:, None], pos_k[None, :]
+    seen = (j <= i) & ((i - j < size) | (j < keep))
+    out = torch.zeros(H, q.shape[0], k.shape[0], dtype=F64)
+    for hd in range(H):
+        s = (q[:, hd] @ k[:, hd // heads_per_kv].T) * scale
+        if cap > 0:
+            s = cap * torch.tanh(s / cap)
+        s = s.masked_fill(~seen, -math.inf)
+        mx = torch.maximum(s.max(-1, keepdim=True).values, sink[hd])
+        e = torch.exp(s - mx)
+        out[hd] = e / (e.sum(-1, keepdim=True) + torch.exp(sink[hd] - mx))
+    return out
+
+
+def mixed_values(weights, talk, v, heads_per_kv: int):
+    """weights [H, Tq, Tk] mixed across heads by talk [H, H]; head h reads the values of its own KV head."""
+    mixed = torch.einsum("hg,gij->hij", talk, weights)
+    return torch.stack([mixed[hd] @ v[:, hd // heads_per_kv] for hd in range(weights.shape[0])], dim=1)
 
 
 def window_attention(h, W, m: dict):
@@ -107,20 +139,9 @@ def window_attention(h, W, m: dict):
     v = short_conv(h @ W["v"].T + W["v.b"], W["v.conv"]).view(t, G, vd)
     q = rotate(q.view(t, H, d), pos, m["rot"], "pairs")
     k = rotate(k.view(t, G, d), pos, m["rot"], "pairs")
-    cap, size, keep = float(m["softcap"]), int(m["mask"]["size"]), int(m["mask"]["keep_first"])
-    i, j = pos[:, None], pos[None, :]
-    seen = (j <= i) & ((i - j < size) | (j < keep))
-    weights = torch.zeros(H, t, t, dtype=F64)
-    for hd in range(H):
-        s = (q[:, hd] @ k[:, hd // (H // G)].T) * float(m["scale"])
-        s = cap * torch.tanh(s / cap)
-        s = s.masked_fill(~seen, -math.inf)
-        mx = torch.maximum(s.max(-1, keepdim=True).values, W["sink"][hd])
-        e = torch.exp(s - mx)
-        weights[hd] = e / (e.sum(-1, keepdim=True) + torch.exp(W["sink"][hd] - mx))
-    mixed = torch.einsum("hg,gij->hij", W["talk"], weights)
-    o = torch.stack([mixed[hd] @ v[:, hd // (H // G)] for hd in range(H)], dim=1)
-    return o.reshape(t, H * vd) @ W["o"].T
+    w = window_weights(q, k, pos, pos, H // G, float(m["scale"]), float(m["softcap"]), int(m["mask"]["size"]),
+                       int(m["mask"]["keep_first"]), W["sink"])
+    return mixed_values(w, W["talk"], v, H // G).reshape(t, H * vd) @ W["o"].T
 
 
 def gated_recurrence(h, W, m: dict, eps: float):
@@ -130,13 +151,7 @@ def gated_recurrence(h, W, m: dict, eps: float):
     q = torch.nn.functional.silu(h @ W["q"].T).view(t, H, d)
     v = (h @ W["v"].T).view(t, H, vd)
     f = (W["lower"] + (1 - W["lower"]) * torch.sigmoid(h @ W["f"].T + W["f.b"])).view(t, H, d)
-    o = torch.zeros(t, H, vd, dtype=F64)
-    for hd in range(H):
-        S = torch.zeros(d, vd, dtype=F64)
-        for i in range(t):
-            S = f[i, hd][:, None] * S + torch.outer(1 - f[i, hd], v[i, hd])
-            o[i, hd] = S.T @ q[i, hd]
-    o = rms_unit(o, eps) * W["norm"]
+    o = rms_unit(linear_recurrence(q, 1 - f, v, f), eps) * W["norm"]
     return o.reshape(t, H * vd) @ W["o"].T
 
 
@@ -265,5 +280,28 @@ def write_checkpoint(path, cfg: dict, weights: dict) -> Path:
     path = Path(path)
     path.mkdir(parents=True, exist_ok=True)
     (path / "config.json").write_text(json.dumps(cfg))
-    save_file({k: v.contiguous() for k, v in weights.items()}, str(path / "model.safetensors"))
+    save_file({k: v.contiguous().clone() for k, v in weights.items()}, str(path / "model.safetensors"))
     return path
+
+
+def greedy(cfg: dict, weights: dict, prompt: list[int], n_new: int) -> list[int]:
+    toks = list(prompt)
+    for _ in range(n_new):
+        logits, _ = forward(cfg, weights, toks)
+        toks.append(int(logits[-1].argmax()))
+    return toks[len(prompt):]
+
+
+def row_errors(got, want):
+    """Per row: rms of the difference (means taken off) over the rms of the wanted row (mean taken off)."""
+    g, w = got.double(), want.double()
+    d = (g - w) - (g - w).mean(-1, keepdim=True)
+    ref = w - w.mean(-1, keepdim=True)
+    return d.pow(2).mean(-1).sqrt() / ref.pow(2).mean(-1).sqrt().clamp_min(1e-30)
+
+
+def check_rows(got, want, tol, what=""):
+    assert got.shape == want.shape, f"{what}: shape {tuple(got.shape)} != {tuple(want.shape)}"
+    err = row_errors(got, want)
+    bad = int(err.argmax())
+    assert err.max().item() < tol, f"{what}: row {bad} is off by {err.max().item():.3g} (allowed {tol})"

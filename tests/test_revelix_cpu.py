@@ -1,0 +1,161 @@
+"""Revelix on the CPU (the PyTorch definitions of the ops, fp32): every mechanism against its float64
+definition, then the engine (scheduler, pages, state slots, batch assembly, model) against the oracle."""
+
+import json
+import os
+import subprocess
+import sys
+import tempfile
+
+import pytest
+import torch
+
+import revelix_cases as rc
+import revelix_oracle as ro
+from vllm_production_stack_amd.engine.block_manager import StateSlots
+from vllm_production_stack_amd.engine.config import ParallelMixerSpec, RetentionSpec, resolve_model
+
+DEV = torch.device("cpu")
+TOL = 2e-5
+
+
+@pytest.fixture(scope="module")
+def model_a():
+    cfg = rc.config_a()
+    return cfg, ro.random_weights(cfg, seed=3)
+
+
+@pytest.fixture(scope="module")
+def model_b():
+    cfg = rc.config_b()
+    return cfg, ro.random_weights(cfg, seed=4)
+
+
+def test_norm_and_activation():
+    rc.case_dyt_and_xielu(DEV, "float32", 1e-5)
+
+
+def test_rotary_tables():
+    rc.case_rotary_tables()
+
+
+def test_recurrences():
+    rc.case_recurrences(DEV, "float32", 1e-5)
+
+
+def test_head_norm():
+    rc.case_head_norm(DEV, "float32", 1e-5)
+
+
+def test_short_convolution():
+    rc.case_short_conv(DEV, "float32", 1e-5)
+
+
+def test_window_edges():
+    rc.case_window_edges(DEV, "float32", 1e-5)
+
+
+def test_far_keys():
+    rc.case_far_keys(DEV, "float32", 1e-5)
+
+
+def test_layers(model_a, model_b):
+    rc.check_layers("cpu", "float32", TOL, *model_a)
+    rc.check_layers("cpu", "float32", TOL, *model_b)
+
+
+def test_whole_decode_and_portions(model_a):
+    # whole; all but the last tokens then one by one; portions of many sizes around page and window borders
+    rc.check_cuts("cpu", "float32", TOL, *model_a, 150, [[150], [118], [64, 64], [63, 2, 63, 2], [2, 2, 2, 58, 1, 64],
+                                                         [1, 1, 1, 25, 23, 2]])
+
+
+def test_other_sizes_and_first_tokens(model_b):
+    rc.check_cuts("cpu", "float32", TOL, *model_b, 140, [[140], [1], [2, 1, 2], [3, 61, 64], [70, 5, 60]])
+    rc.check_cuts("cpu", "float32", TOL, *model_b, 1, [[1]])
+    rc.check_cuts("cpu", "float32", TOL, *model_b, 3, [[3], [1, 2]])
+
+
+def test_long_decode(model_b):
+    rc.check_cuts("cpu", "float32", TOL, *model_b, 330, [[20]], pages=6)  # 310 single tokens over five pages
+
+
+def test_batches_and_reuse(model_a):
+    rc.check_batches("cpu", "float32", TOL, *model_a)
+
+
+def test_greedy_generation(model_a, model_b):
+    rc.check_generate("cpu", "float32", *model_a)
+    rc.check_generate("cpu", "float32", *model_b)
+
+
+def test_preempted_sequences_start_over(model_a):
+    rc.check_preemption("cpu", "float32", *model_a)
+
+
+def test_state_slots():
+    s = StateSlots(2)
+    a, b = s.take(), s.take()
+    assert {a, b} == {0, 1} and s.num_free() == 0
+    with pytest.raises(MemoryError):
+        s.take()
+    s.give_back(a)
+    assert s.take() == a
+
+
+def test_config_reader_and_loader_refusals(model_a):
+    cfg, w = model_a
+    folder = ro.write_checkpoint(tempfile.mkdtemp(prefix="rx-"), cfg, w)
+    mc, path = resolve_model(str(folder))
+    assert mc.architecture == "revelix" and len(mc.layer_specs) == 3 and mc.tie_word_embeddings
+    assert isinstance(mc.layer_specs[0].mixer, RetentionSpec) and isinstance(mc.layer_specs[1].mixer, ParallelMixerSpec)
+    left = mc.layer_specs[1].mixer.left
+    assert (left.window, left.keep_first, left.conv, left.rot.layout, left.rot.scaling) == (24, 3, 3, "pairs", (4.0, 64.0, 16.0, 1.0))
+    assert mc.layer_specs[0].mixer.rot.layout == "half" and mc.logit_scale == 0.7
+    assert 0.95 < mc.num_params() / sum(v.numel() for v in w.values()) <= 1.0  # matrices only
+    from vllm_production_stack_amd.models.loader import build_model
+
+    for broken in ("missing", "extra", "shape"):
+        w2 = dict(w)
+        if broken == "missing":
+            del w2["l1.mix.left.sink"]
+        elif broken == "extra":
+            w2["l0.mix.left.q"] = w["l1.mix.left.q"]
+        else:
+            w2["l2.mix.o"] = w["l2.mix.o"][:, :-1].contiguous()
+        bad = ro.write_checkpoint(tempfile.mkdtemp(prefix="rx-"), cfg, w2)
+        with pytest.raises(ValueError):
+            build_model(mc, torch.float32, DEV, 256, bad)
+    for key, value in (("type", "retentive"), ("mlp", {"kind": "moe", "ff": 8})):
+        c2 = json.loads(json.dumps(cfg))
+        c2["layers"][0][key] = value
+        (folder / "config.json").write_text(json.dumps(c2))
+        with pytest.raises(ValueError):
+            resolve_model(str(folder))
+
+
+def test_replay_command(model_b):
+    """bin/trace_run on a checkpoint: steps on stdin, logits files and 'done' lines out."""
+    cfg, w = model_b
+    folder = ro.write_checkpoint(tempfile.mkdtemp(prefix="rx-"), cfg, w)
+    out = tempfile.mkdtemp(prefix="rx-out-")
+    a, b = rc.tokens(cfg, 70, 1), rc.tokens(cfg, 9, 2)
+    steps = [{"step": 0, "entries": [{"id": "a", "tokens": a[:66], "want": [0, 65]}], "end": []},
+             {"step": 1, "entries": [{"id": "a", "tokens": a[66:67], "want": []}, {"id": "b", "tokens": b, "want": [8]}], "end": ["b"]},
+             {"step": 2, "entries": [{"id": "a", "tokens": a[67:], "want": [2]}], "end": ["a"]}]
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    p = subprocess.run([sys.executable, os.path.join(root, "bin", "trace_run"), "--model", str(folder), "--dtype", "float32",
+                        "--out", out, "--max-tokens", "192", "--device", "cpu"],
+                       input="\n".join(json.dumps(s) for s in steps) + "\n", capture_output=True, text=True, timeout=300)
+    assert p.returncode == 0, p.stderr[-2000:]
+    assert [ln for ln in p.stdout.splitlines() if ln.startswith("done")] == ["done 0", "done 1", "done 2"]
+    assert not os.path.exists(os.path.join(out, "1.f32")) or os.path.getsize(os.path.join(out, "1.f32")) == 4 * cfg["vocab"]
+    la, lb = ro.forward(cfg, w, a)[0], ro.forward(cfg, w, b)[0]
+    import numpy as np
+
+    got0 = torch.from_numpy(np.fromfile(os.path.join(out, "0.f32"), dtype="<f4").reshape(2, -1))
+    got1 = torch.from_numpy(np.fromfile(os.path.join(out, "1.f32"), dtype="<f4").reshape(1, -1))
+    got2 = torch.from_numpy(np.fromfile(os.path.join(out, "2.f32"), dtype="<f4").reshape(1, -1))
+    ro.check_rows(got0, la[[0, 65]], TOL, "step 0")
+    ro.check_rows(got1, lb[[8]], TOL, "step 1")
+    ro.check_rows(got2, la[[69]], TOL, "step 2")

@@ -590,7 +590,8 @@ def window_attention(q, pool, cache_off, kv_heads, vdim, block_tables, row_seq, 
         kk = kc[pages, idx % PAGE].float()       # [keys, kv_heads, dim]
         vv = vc[pages, idx % PAGE].float()       # [keys, kv_heads, vdim]
         sc = torch.einsum("hd,khd->hk", q[r].float(), kk.repeat_interleave(rep, dim=1)) * scale
-        sc = softcap * torch.tanh(sc / softcap)
+        if softcap > 0:
+            sc = softcap * torch.tanh(sc / softcap)
         mx = torch.maximum(sc.max(-1).values, sink)
         e = torch.exp(sc - mx[:, None])
         w = e / (e.sum(-1) + torch.exp(sink - mx))[:, None]
