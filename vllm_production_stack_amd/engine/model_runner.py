@@ -727,8 +727,9 @@ class ModelRunner:
         """A prefill part that a captured graph can hold: one rank, no adapters, no pooling, at most
         ``_PREFILL_GRAPH_SEQS`` sequences and the largest row bucket."""
         if (not prefills or self.distributed or len(prefills) > _PREFILL_GRAPH_SEQS
-                or sum(s.n for s in prefills) > _PREFILL_ROW_BUCKETS[-1] or hasattr(self.model, "plan_prefill")):
-            return False  # (a model with a prefill work list of its own builds it per step, on the host)
+                or sum(s.n for s in prefills) > _PREFILL_ROW_BUCKETS[-1] or hasattr(self.model, "plan_prefill")
+                or hasattr(self.model, "plan_batch")):
+            return False  # (a model with a work list or batch description of its own builds it per step, on the host)
         lora = self.model.lora is not None
         return not any(s.req.pooling or (lora and s.req.lora_slot >= 0) for s in prefills)
 
@@ -963,7 +964,7 @@ class ModelRunner:
         for b in sorted(todo, reverse=True):
             self._graphs[b] = self._capture(b)
         n = len(todo)
-        if not self.distributed and not hasattr(self.model, "plan_prefill"):
+        if not self.distributed and not hasattr(self.model, "plan_prefill") and not hasattr(self.model, "plan_batch"):
             for rows in reversed(_PREFILL_ROW_BUCKETS):  # the small prefill parts of mixed steps
                 if rows <= self.cfg.max_num_batched_tokens and rows not in self._prefill_graphs:
                     self._prefill_graphs[rows] = self._capture_prefill(rows)
