@@ -1,6 +1,6 @@
 """Prefill and decode throughput of one decoder design beside the closest existing one at equal size.
 
-    python bench.py --arch-compare zururax [--arch-sizes s,m] [--arch-prompt 4096] [--arch-batch 32]
+    python bench.py --arch-compare zururax|revelix [--arch-sizes s,m] [--arch-prompt 4096] [--arch-batch 32]
 
 Random weights at layer shapes of real models (a few layers each); both models run through the same
 engine (scheduler, paged pool, HIP-graph decode).  Prefill: prompts of --arch-prompt tokens in chunks of
@@ -28,6 +28,8 @@ def _configs(design: str, size: str):
     from vllm_production_stack_amd.engine.config import ModelConfig, zururax_config
 
     z = SIZES[size]
+    if design == "revelix":
+        return _revelix_configs(size)
     if design != "zururax":
         raise SystemExit(f"--arch-compare: unknown design {design!r}")
 
@@ -51,6 +53,35 @@ def _configs(design: str, size: str):
                       intermediate_size=z["ff"], num_layers=z["layers"], num_heads=z["heads"],
                       num_kv_heads=max(1, z["heads"] // 4), head_dim=128, num_experts=z["experts"],
                       num_experts_per_tok=z["top"], max_position_embeddings=32768)
+    return new, old
+
+
+def _revelix_configs(size: str):
+    """Revelix (retention | parallel | parallel | retention, every layer with a feed-forward of four times the
+    width) beside the closest existing design: a dense grouped-query decoder of the same width, depth, heads
+    and feed-forward parameter count."""
+    from vllm_production_stack_amd.engine.config import ModelConfig, revelix_config
+
+    z = SIZES[size]
+    w, heads = z["width"], z["heads"]
+    ff = 4 * w
+    mlp = {"kind": "dense", "ff": ff}
+    retention = {"type": "retention", "mlp": mlp,
+                 "mixer": {"heads": heads, "dim": 128, "vdim": 256, "rot": {"base": 10000.0, "dims": 128},
+                           "decay": [1 - 2.0 ** (-5 - 3 * i / heads) for i in range(heads)]}}
+    parallel = {"type": "parallel", "mlp": mlp,
+                "mixer": {"left": {"heads": heads, "kv_heads": heads // 4, "dim": 128, "vdim": 128, "conv": 4,
+                                   "mask": {"size": 1024, "keep_first": 4},
+                                   "rot": {"base": 1e6, "dims": 128,
+                                           "scaling": {"factor": 8.0, "original": 4096, "fast": 32.0, "slow": 1.0}},
+                                   "scale": 128 ** -0.5, "softcap": 50.0},
+                          "right": {"heads": heads // 2, "dim": 128, "vdim": 128},
+                          "left_scale": 0.7, "right_scale": 0.7}}
+    new = revelix_config(f"revelix-{size}", VOCAB, w, [retention, parallel, parallel, retention], logit_scale=0.5,
+                         max_position_embeddings=32768)
+    old = ModelConfig(name=f"llama-{size}", architecture="llama", vocab_size=VOCAB, hidden_size=w,
+                      intermediate_size=(2 * ff // 3 + 255) // 256 * 256, num_layers=4, num_heads=heads,
+                      num_kv_heads=heads // 4, head_dim=128, max_position_embeddings=32768)
     return new, old
 
 

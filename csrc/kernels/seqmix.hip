@@ -252,7 +252,7 @@ __global__ __launch_bounds__(256) void short_conv_qkv_kernel(
   const int nq = heads * dim, nk = kv_heads * dim, nv = kv_heads * vdim;
   const long kv_slot = slots[row];
   T* kdst = kv_slot >= 0 ? cache + (kv_slot / PAGE) * page_stride + (kv_slot % PAGE) * (long)nk : nullptr;
-  T* vdst = kv_slot >= 0 ? cache + (kv_slot / PAGE) * page_stride + (long)PAGE * nk + (kv_slot % PAGE) * (long)nv : nullptr;
+  T* vdst = kv_slot >= 0 ? cache + (kv_slot / PAGE) * page_stride + (long)PAGE * nk + (kv_slot % PAGE) : nullptr;  // V^T
   for (int c = threadIdx.x; c < chans; c += 256) {
     if (c < nq + nk) {
       const int base = c < nq ? (c / dim) * dim : nq + ((c - nq) / dim) * dim;
@@ -261,7 +261,7 @@ __global__ __launch_bounds__(256) void short_conv_qkv_kernel(
       if (c < nq) Cv<T>::st(q_out + row * nq + c, r);
       else if (kdst) Cv<T>::st(kdst + (c - nq), r);
     } else if (vdst) {
-      Cv<T>::st(vdst + (c - nq - nk), ys[c]);
+      Cv<T>::st(vdst + (long)(c - nq - nk) * PAGE, ys[c]);
     }
   }
 }
@@ -292,9 +292,28 @@ __global__ __launch_bounds__(256) void conv_tail_kernel(const T* __restrict__ pr
 }
 
 // ---------------------------------------------------------------------------------
-// One workgroup per (row, query head): 256 keys per step.  Layer cache inside a page: K [PAGE][kv_heads * dim],
-// then V [PAGE][kv_heads * vdim].  out [rows, heads, kv_heads, vdim] fp32: the head's softmax weights applied
-// to the values of every KV head (the head mixing that follows needs them).
+// Layer cache inside a page: K [PAGE][kv_heads * dim], then V transposed [kv_heads * vdim][PAGE].
+// The pages a query at position p (or a tile of queries p_a .. p_b) has to visit: those that hold kept first
+// tokens below the window, then the window's own; the mask decides key by key.
+struct PageWalk {
+  int n_keep, first, count;
+  __device__ __forceinline__ PageWalk(int pa, int pb, int window, int keep_first) {
+    const int lo = max(0, pa - window + 1);
+    first = lo / PAGE;
+    n_keep = min((min(keep_first, lo) + PAGE - 1) / PAGE, first);
+    count = n_keep + pb / PAGE - first + 1;
+  }
+  __device__ __forceinline__ int page(int i) const { return i < n_keep ? i : first + (i - n_keep); }
+};
+
+__device__ __forceinline__ bool key_seen(int j, int p, int window, int keep_first) {
+  return j <= p && (p - j < window || j < keep_first);
+}
+
+// Plain kernel, every size and both dtypes.  One workgroup per (row, query head), four pages per step: a thread
+// scores one key, then owns value channels and walks the step's keys in runs of 16 bytes.
+// out [rows, heads, kv_heads, vdim] fp32: the head's softmax weights applied to the values of every KV head
+// (the head mixing that follows needs them).
 constexpr int WA_KEYS = 256;
 constexpr int WA_ACC = 8;  // kv_heads * vdim <= 256 * WA_ACC
 
@@ -307,7 +326,8 @@ __global__ __launch_bounds__(256) void window_attention_kernel(
   extern __shared__ float sm[];
   __shared__ float red[4];
   __shared__ float ps[WA_KEYS];
-  __shared__ long voff[WA_KEYS];
+  __shared__ long pbase[WA_KEYS / PAGE];
+  constexpr int RUN = 16 / sizeof(T);  // keys per 16-byte load of a V^T row
   const long row = blockIdx.x;
   const int head = blockIdx.y;
   const int tid = threadIdx.x;
@@ -317,56 +337,234 @@ __global__ __launch_bounds__(256) void window_attention_kernel(
   const int nk = kv_heads * dim, nv = kv_heads * vdim;
   float* qs = sm;
   for (int i = tid; i < dim; i += 256) qs[i] = Cv<T>::ld(q + row * q_stride + head * dim + i);
-  const int lo = max(0, pos - window + 1);
-  const int nkeep = min(keep_first, lo);
-  const int total = nkeep + (pos - lo + 1);
+  const PageWalk walk(pos, pos, window, keep_first);
   const int* bt = block_tables + (long)seq * bt_stride;
   float m = sink ? sink[head] : -INFINITY, l = sink ? 1.f : 0.f;
   float acc[WA_ACC];
 #pragma unroll
   for (int a = 0; a < WA_ACC; ++a) acc[a] = 0.f;
   __syncthreads();
-  for (int k0 = 0; k0 < total; k0 += WA_KEYS) {
-    const int kk = k0 + tid;
+  for (int p0 = 0; p0 < walk.count; p0 += WA_KEYS / PAGE) {
+    const int pi = p0 + tid / PAGE, r = tid % PAGE;
     float s = -INFINITY;
-    long off = 0;
-    if (kk < total) {
-      const int j = kk < nkeep ? kk : lo + (kk - nkeep);
-      const long page = (long)bt[j / PAGE] * page_stride;
-      off = page + (long)PAGE * nk + (long)(j % PAGE) * nv;  // the key's value row
-      const T* kp = cache + page + (long)(j % PAGE) * nk + g * dim;
-      float d = 0.f;
-      for (int i = 0; i < dim; ++i) d = fmaf(qs[i], Cv<T>::ld(kp + i), d);
-      d *= scale;
-      s = softcap > 0.f ? softcap * tanhf(d / softcap) : d;
+    if (pi < walk.count) {
+      const int pg = walk.page(pi);
+      const long base = (long)bt[pg] * page_stride;
+      if (r == 0) pbase[tid / PAGE] = base;
+      const int j = pg * PAGE + r;
+      if (key_seen(j, pos, window, keep_first)) {
+        const T* kp = cache + base + (long)r * nk + g * dim;
+        float d = 0.f;
+        for (int i = 0; i < dim; ++i) d = fmaf(qs[i], Cv<T>::ld(kp + i), d);
+        d *= scale;
+        s = softcap > 0.f ? softcap * tanhf(d / softcap) : d;
+      }
     }
     const float mb = blk_max(s, red);
     const float mn = fmaxf(m, mb);
-    const float p = kk < total ? expf(s - mn) : 0.f;
-    const float corr = expf(m - mn);  // 0 while nothing has been seen (m = -inf without a sink)
+    const bool dead = mn == -INFINITY;  // nothing seen so far (no sink) and nothing visible in this step
+    const float p = (dead || s == -INFINITY) ? 0.f : expf(s - mn);
+    const float corr = (dead || m == -INFINITY) ? 0.f : expf(m - mn);
     ps[tid] = p;
-    voff[tid] = off;
-    const float bs = blk_sum(p, red);  // its barriers also publish ps / voff
+    const float bs = blk_sum(p, red);  // its barriers also publish ps / pbase
     l = l * corr + bs;
-    const int nb = min(WA_KEYS, total - k0);
+    const int np = min(WA_KEYS / PAGE, walk.count - p0);
 #pragma unroll
     for (int a = 0; a < WA_ACC; ++a) {
       const int c = a * 256 + tid;
       if (c < nv) {
         float x = acc[a] * corr;
-        for (int k = 0; k < nb; ++k) x = fmaf(ps[k], Cv<T>::ld(cache + voff[k] + c), x);
+        for (int pp = 0; pp < np; ++pp) {
+          const T* vp = cache + pbase[pp] + (long)PAGE * nk + (long)c * PAGE;
+          for (int k = 0; k < PAGE; k += RUN) {
+            T v[RUN];
+            *reinterpret_cast<u32x4*>(v) = *reinterpret_cast<const u32x4*>(vp + k);
+#pragma unroll
+            for (int e = 0; e < RUN; ++e) x = fmaf(ps[pp * PAGE + k + e], (float)v[e], x);
+          }
+        }
         acc[a] = x;
       }
     }
     m = mn;
     __syncthreads();
   }
-  const float inv = 1.f / l;
+  const float inv = l > 0.f ? 1.f / l : 0.f;
 #pragma unroll
   for (int a = 0; a < WA_ACC; ++a) {
     const int c = a * 256 + tid;
     if (c < nv) out[(row * heads + head) * (long)nv + c] = acc[a] * inv;
   }
+}
+
+// Matrix-core kernel (bf16; DIM channels per key, VALL = kv_heads * vdim value channels).  A workgroup takes a
+// tile of up to 64 query slots = (row, query head of ONE key/value group) pairs of consecutive rows of one
+// sequence, so all its slots score against the same keys; wave w owns slots 16 w .. 16 w + 15 end to end
+// (queries as B operands, the [16 x VALL] output in registers).  Per visited page the workgroup stages
+//   K image   [64 keys][DIM]   (+16 B row padding): A operand of S^T = K Q^T
+//   V^T image [VALL][64 keys]  (+16 B row padding): A operand of O^T = V^T P^T   (the page stores V transposed)
+// with 16-byte copies.  The rows of a 16-key score tile are taken from the K image in the order that leaves a
+// lane with 8 consecutive keys per 32 (v_mfma 16x16x32: lane = slot l % 16, rows 4 (l / 16) + e), so the
+// probabilities go from the first product's accumulators into the second without leaving the lane.
+// Scores are capped, masked by window / kept first tokens and normalised online in fp32; a sink logit starts
+// the running state (max = sink, sum = 1).  The next page's loads are in flight while a page is multiplied.
+template <int DIM, int VALL>
+__global__ __launch_bounds__(256) void window_mfma_kernel(
+    const uint16_t* __restrict__ q, long q_stride, const uint16_t* __restrict__ cache, long page_stride,
+    const int* __restrict__ block_tables, int bt_stride, const int* __restrict__ tiles,
+    const int* __restrict__ positions, const float* __restrict__ sink, float* __restrict__ out, int heads, int kv_heads,
+    int window, int keep_first, float scale, float softcap) {
+  constexpr int KS = DIM / 32;
+  constexpr int DT = VALL / 16;
+  constexpr int PK = DIM * 2 + 16;
+  constexpr int PV = PAGE * 2 + 16;
+  constexpr int KB = DIM * PAGE / 8 / 256;   // 16-byte chunks of the K tile per thread
+  constexpr int VB = VALL * PAGE / 8 / 256;  // and of the V^T tile
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+  char* kimg = lds;
+  char* vimg = lds + PAGE * PK;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int c16 = lane & 15, g = lane >> 4;
+  const int group = blockIdx.y, rep = heads / kv_heads;
+  int seq, row0, n_rows, pos0;
+  if (tiles) {
+    const int* e = tiles + 4 * blockIdx.x;
+    seq = e[0], row0 = e[1], n_rows = e[2], pos0 = e[3];
+  } else {  // decode rows: row r is sequence r
+    seq = row0 = blockIdx.x, n_rows = 1, pos0 = positions[blockIdx.x];
+  }
+  if (seq < 0) return;
+  const int n_slots = n_rows * rep;
+  const int slot = wave * 16 + c16;
+  const bool valid = slot < n_slots;
+  const bool wave_active = wave * 16 < n_slots;  // wave-uniform
+  const int tok = valid ? slot / rep : 0;
+  const int head = group * rep + (valid ? slot % rep : 0);
+  const long row = row0 + tok;
+  const int my_pos = valid ? pos0 + tok : -1;
+  const PageWalk walk(pos0, pos0 + n_rows - 1, window, keep_first);
+  const int* bt = block_tables + (long)seq * bt_stride;
+  const long k_off = (long)group * DIM, k_row = (long)kv_heads * DIM, v_off = (long)PAGE * kv_heads * DIM;
+
+  bf16x8 qf[KS];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) {
+    u32x4 v = {0u, 0u, 0u, 0u};
+    if (valid) v = *reinterpret_cast<const u32x4*>(q + row * q_stride + (long)head * DIM + 32 * ks + 8 * g);
+    qf[ks] = __builtin_bit_cast(bf16x8, v);
+  }
+  float m = (sink && valid) ? sink[head] : -INFINITY;
+  float l = (sink && valid) ? 1.f : 0.f;
+  f32x4 o[DT];
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt) o[dt] = (f32x4){0.f, 0.f, 0.f, 0.f};
+
+  u32x4 kb[KB], vb[VB];
+  auto fetch = [&](int i) {
+    const uint16_t* src = cache + (long)bt[walk.page(i)] * page_stride;
+#pragma unroll
+    for (int b = 0; b < KB; ++b) {
+      const int id = tid + 256 * b, dc = id % (DIM / 8), key = id / (DIM / 8);
+      kb[b] = *reinterpret_cast<const u32x4*>(src + key * k_row + k_off + 8 * dc);
+    }
+#pragma unroll
+    for (int b = 0; b < VB; ++b) vb[b] = *reinterpret_cast<const u32x4*>(src + v_off + (long)(tid + 256 * b) * 8);
+  };
+  auto stash = [&]() {
+#pragma unroll
+    for (int b = 0; b < KB; ++b) {
+      const int id = tid + 256 * b, dc = id % (DIM / 8), key = id / (DIM / 8);
+      *reinterpret_cast<u32x4*>(kimg + key * PK + 16 * dc) = kb[b];
+    }
+#pragma unroll
+    for (int b = 0; b < VB; ++b) {
+      const int id = tid + 256 * b;
+      *reinterpret_cast<u32x4*>(vimg + (id >> 3) * PV + 16 * (id & 7)) = vb[b];
+    }
+  };
+  // K image row of score-tile row c16 in tile nt: key 32 (nt / 2) + 8 (c16 / 4) + 4 (nt % 2) + c16 % 4
+  int krow[4];
+#pragma unroll
+  for (int nt = 0; nt < 4; ++nt) krow[nt] = (32 * (nt >> 1) + 8 * (c16 >> 2) + 4 * (nt & 1) + (c16 & 3)) * PK + 16 * g;
+  const float inv_cap = softcap > 0.f ? 1.f / softcap : 0.f;
+
+  if (walk.count > 0) fetch(0);
+  for (int i = 0; i < walk.count; ++i) {
+    __syncthreads();  // the previous page's fragment reads are done
+    stash();
+    __syncthreads();
+    if (i + 1 < walk.count) fetch(i + 1);
+    if (!wave_active) continue;
+    const int j0 = walk.page(i) * PAGE;
+    f32x4 s[4];
+#pragma unroll
+    for (int nt = 0; nt < 4; ++nt) s[nt] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+      for (int nt = 0; nt < 4; ++nt) {
+        const bf16x8 a = *reinterpret_cast<const bf16x8*>(kimg + krow[nt] + 64 * ks);
+        s[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qf[ks], s[nt], 0, 0, 0);
+      }
+    float mx = -INFINITY;
+#pragma unroll
+    for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int j = j0 + 32 * (nt >> 1) + 8 * g + 4 * (nt & 1) + e;
+        float v = -INFINITY;
+        if (key_seen(j, my_pos, window, keep_first)) {
+          v = s[nt][e] * scale;
+          if (softcap > 0.f) {  // cap * tanh(v / cap), tanh(x) = 1 - 2 / (exp(2 x) + 1)
+            const float x = v * inv_cap;
+            v = softcap * (1.f - 2.f / (__expf(2.f * x) + 1.f));
+          }
+        }
+        s[nt][e] = v;
+        mx = fmaxf(mx, v);
+      }
+    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const float mn = fmaxf(m, mx);
+    const bool dead = mn == -INFINITY;
+    const float corr = (dead || m == -INFINITY) ? (dead ? 1.f : 0.f) : __expf(m - mn);
+    float psum = 0.f;
+#pragma unroll
+    for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const float pv = dead ? 0.f : __expf(s[nt][e] - mn);
+        s[nt][e] = pv;
+        psum += pv;
+      }
+    psum += __shfl_xor(psum, 16, 64);
+    psum += __shfl_xor(psum, 32, 64);
+    l = l * corr + psum;
+    m = mn;
+    bf16x8 pf[2];
+#pragma unroll
+    for (int kk = 0; kk < 2; ++kk) {
+      u32x4 w = {pack_bf16x2(s[2 * kk][0], s[2 * kk][1]), pack_bf16x2(s[2 * kk][2], s[2 * kk][3]),
+                 pack_bf16x2(s[2 * kk + 1][0], s[2 * kk + 1][1]), pack_bf16x2(s[2 * kk + 1][2], s[2 * kk + 1][3])};
+      pf[kk] = __builtin_bit_cast(bf16x8, w);
+    }
+    if (!__all(corr == 1.f)) {
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) o[dt] *= corr;
+    }
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int kk = 0; kk < 2; ++kk) {
+        const bf16x8 a = *reinterpret_cast<const bf16x8*>(vimg + (16 * dt + c16) * PV + 16 * (4 * kk + g));
+        o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pf[kk], o[dt], 0, 0, 0);
+      }
+  }
+  if (!valid) return;
+  const float inv = l > 0.f ? 1.f / l : 0.f;
+  float* dst = out + (row * heads + head) * (long)VALL + 4 * g;
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt) *reinterpret_cast<f32x4*>(dst + 16 * dt) = o[dt] * inv;
 }
 
 template <typename T>
@@ -492,6 +690,50 @@ VPSA_EXPORT int vpsa_window_attention(const void* q, long q_stride, const void* 
                       (const T*)q, q_stride, (const T*)cache, page_stride, block_tables, bt_stride, row_seq, positions,
                       sink, out, heads, kv_heads, dim, vdim, window, keep_first, scale, softcap)));
   return 0;
+}
+
+VPSA_EXPORT int vpsa_window_mfma_supported(int heads, int kv_heads, int dim, int vdim) {
+  const int vall = kv_heads * vdim;
+  return (dim == 64 || dim == 128) && (vall == 128 || vall == 256 || vall == 512) && heads % kv_heads == 0 &&
+         heads / kv_heads <= 64;
+}
+
+template <int DIM, int VALL>
+static int launch_window_mfma(const void* q, long q_stride, const void* cache, long page_stride, const int* block_tables,
+                              int bt_stride, const int* tiles, const int* positions, const float* sink, float* out,
+                              int n_tiles, int heads, int kv_heads, int window, int keep_first, float scale,
+                              float softcap, hipStream_t st) {
+  constexpr int LDS = PAGE * (DIM * 2 + 16) + VALL * (PAGE * 2 + 16);
+  static bool attr_set = false;
+  if (!attr_set) {
+    if (hipFuncSetAttribute((const void*)window_mfma_kernel<DIM, VALL>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                            LDS) != hipSuccess)
+      return -2;
+    attr_set = true;
+  }
+  window_mfma_kernel<DIM, VALL><<<dim3(n_tiles, kv_heads), dim3(256), LDS, st>>>(
+      (const uint16_t*)q, q_stride, (const uint16_t*)cache, page_stride, block_tables, bt_stride, tiles, positions, sink,
+      out, heads, kv_heads, window, keep_first, scale, softcap);
+  return 0;
+}
+
+// tiles: int32 [n_tiles][4] = (sequence, first row, rows, position of the first row), -1 sequence = skip;
+// nullptr: n_tiles decode rows, row r = sequence r at positions[r].
+VPSA_EXPORT int vpsa_window_attention_mfma(const void* q, long q_stride, const void* cache, long page_stride,
+                                           const int* block_tables, int bt_stride, const int* tiles,
+                                           const int* positions, const float* sink, float* out, int n_tiles, int heads,
+                                           int kv_heads, int dim, int vdim, int window, int keep_first, float scale,
+                                           float softcap, hipStream_t stream) {
+  if (n_tiles <= 0) return 0;
+  if (!vpsa_window_mfma_supported(heads, kv_heads, dim, vdim)) return 2;
+  const int vall = kv_heads * vdim;
+#define WM(D, V)                                                                                                      \
+  if (dim == D && vall == V)                                                                                          \
+    return launch_window_mfma<D, V>(q, q_stride, cache, page_stride, block_tables, bt_stride, tiles, positions, sink,  \
+                                    out, n_tiles, heads, kv_heads, window, keep_first, scale, softcap, stream);
+  WM(64, 128) WM(64, 256) WM(64, 512) WM(128, 128) WM(128, 256) WM(128, 512)
+#undef WM
+  return 2;
 }
 
 VPSA_EXPORT int vpsa_mix_heads(const float* u, const float* talk, void* y, int rows, int heads, int kv_heads, int vdim,

@@ -250,6 +250,51 @@ def case_far_keys(dev, dtype, tol):
         close(ops.mix_heads(u, torch.eye(heads).to(dev), torch.float32).view(len(rows), heads, vdim), want, tol, "far keys")
 
 
+def case_window_tiles(dev, heads, kv_heads, dim, vdim, size, keep, tol=2e-2):
+    """The matrix-core kernel (bf16): chunks of consecutive rows of two sequences as tiles, and single
+    rows as a decode batch; every row looks for one key at an edge of what it may see."""
+    dt = torch.bfloat16
+    g = torch.Generator().manual_seed(6)
+    rep = heads // kv_heads
+    assert ops.window_mfma_supported(heads, kv_heads, dim, vdim)
+    cap, scale = 15.0, 1.0
+    n_keys = 330
+    order = [4, 1, 6, 0, 3, 7]
+    k, v, pool, off = _window_setup(dev, dt, heads, kv_heads, dim, vdim, n_keys, g, order)
+    talk = (torch.eye(heads) * 0.8 + 0.2 * torch.randn(heads, heads, generator=g))
+    sink = torch.randn(heads, generator=g)
+    chunks = [(0, 150, 180), (1, 0, 70), (2, 325, 5)]       # (block-table row = sequence of the batch, first position, rows)
+    bt = i32([order, order, order], dev)
+    pos_q, seqs = [], []
+    for sq, p0, n in chunks:
+        pos_q += list(range(p0, p0 + n))
+        seqs += [sq] * n
+    t = len(pos_q)
+    q = torch.randn(t, heads, dim, generator=g) * 0.05
+    targets = []
+    for r, p in enumerate(pos_q):
+        cand = [j for j in (p, p - 1, p - size + 1, p - size, keep - 1, keep, 0, 63, 64, 127, 128, p - size // 2) if 0 <= j <= p]
+        j = cand[r % len(cand)]
+        targets.append(j)
+        q[r] += 30.0 * k[j, torch.arange(heads) // rep].float() / dim
+    q = q.to(dt)
+    pq = torch.tensor(pos_q)
+    w = ro.window_weights(q.double(), k.double(), pq, torch.arange(n_keys), rep, scale, cap, size, keep, sink.double())
+    want = ro.mixed_values(w, talk.double(), v.double(), rep)
+    tiles = torch.from_numpy(ops.build_window_tiles([n for _, _, n in chunks], [p0 + n for _, p0, n in chunks], heads,
+                                                    kv_heads)).to(dev)
+    u = ops.window_attention(q.to(dev), pool, off, kv_heads, vdim, bt, i32(seqs, dev), i32(pos_q, dev), size, keep, scale,
+                             cap, sink.to(dev), tiles=tiles)
+    plain = ops.window_attention(q.to(dev), pool, off, kv_heads, vdim, bt, i32(seqs, dev), i32(pos_q, dev), size, keep,
+                                 scale, cap, sink.to(dev))
+    close(ops.mix_heads(plain, talk.to(dev), torch.float32).view(t, heads, vdim), want, 2e-5, "plain kernel")
+    close(ops.mix_heads(u, talk.to(dev), torch.float32).view(t, heads, vdim), want, tol, "tiles")
+    rows = list(range(0, t, 7))
+    u = ops.window_attention(q[rows].to(dev), pool, off, kv_heads, vdim, i32([order] * len(rows), dev), None,
+                             i32([pos_q[r] for r in rows], dev), size, keep, scale, cap, sink.to(dev))
+    close(ops.mix_heads(u, talk.to(dev), torch.float32).view(len(rows), heads, vdim), want[rows], tol, "decode rows")
+
+
 def case_short_conv(dev, dtype, tol):
     """Convolution + rotation + cache write: whole against portions shorter than the taps, a restart in
     a slot that held something else, two sequences in one launch."""

@@ -56,6 +56,13 @@ def test_window_edges(dtype):
     rc.case_far_keys(DEV, dtype, 2e-5)
 
 
+@pytest.mark.parametrize("heads,kv_heads,dim,vdim,size,keep", [(4, 2, 64, 64, 70, 3), (8, 2, 128, 128, 100, 0),
+                                                                (3, 1, 64, 128, 64, 65), (16, 4, 128, 128, 129, 4),
+                                                                (4, 4, 128, 64, 1000, 2)])
+def test_window_attention_on_the_matrix_cores(heads, kv_heads, dim, vdim, size, keep):
+    rc.case_window_tiles(DEV, heads, kv_heads, dim, vdim, size, keep)
+
+
 @pytest.mark.parametrize("dtype,tol", MODES)
 def test_layers(dtype, tol, model_a, model_b):
     rc.check_layers("cuda", dtype, tol, *model_a)

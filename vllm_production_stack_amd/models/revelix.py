@@ -203,6 +203,14 @@ class RevelixModel:
         meta.row_seq = to_dev(seq, torch.int32)
         if plan["num_prefill"]:
             meta.pre_row_seq = to_dev([s - nd for s in seq[nd:]], torch.int32)
+            meta.pre_win_tiles = {}
+            if self.device.type == "cuda" and self.dtype == torch.bfloat16:
+                for key in sorted({(s.mixer.left.heads, s.mixer.left.kv_heads) for s in self.specs
+                                   if isinstance(s.mixer, ParallelMixerSpec)
+                                   and ops.window_mfma_supported(s.mixer.left.heads, s.mixer.left.kv_heads,
+                                                                 s.mixer.left.dim, s.mixer.left.vdim)}):
+                    tiles = ops.build_window_tiles(plan["q_lens"], plan["pre_ctx"], *key)
+                    meta.pre_win_tiles[key] = torch.from_numpy(tiles).pin_memory().to(self.device, non_blocking=True)
 
     def plan_decode_graph(self, meta: BatchMeta, bsz: int, state_slots: torch.Tensor) -> None:
         """The same for a captured decode step of ``bsz`` rows: ``state_slots`` is a graph input."""
@@ -236,7 +244,7 @@ class RevelixModel:
         if meta.num_prefill_seqs > 0:
             ops.window_attention(q[nd:], pool, lw.cache_off, a.kv_heads, a.vdim, meta.pre_block_tables,
                                  meta.pre_row_seq, meta.positions[nd:], a.window, a.keep_first, a.scale, a.softcap,
-                                 lw.sink, out=u[nd:])
+                                 lw.sink, out=u[nd:], tiles=(meta.pre_win_tiles or {}).get((a.heads, a.kv_heads)))
         left = ops.linear(ops.mix_heads(u, lw.talk, self.dtype), lw.w_o)
         c0 = a.channels
         rd = r.heads * r.dim

@@ -42,7 +42,7 @@ def _kernels():
             "vpsa_gather_rows", "vpsa_moe_finish", "vpsa_latent_mfma_supported", "vpsa_latent_attention_mfma",
             "vpsa_moe_mfma_act",
             "vpsa_add_dyt", "vpsa_recurrent_scan", "vpsa_head_rms", "vpsa_short_conv_qkv", "vpsa_window_attention",
-            "vpsa_mix_heads", "vpsa_xielu",
+            "vpsa_mix_heads", "vpsa_xielu", "vpsa_window_mfma_supported", "vpsa_window_attention_mfma",
         ):
             getattr(lib, name).restype = c_int
         lib.vpsa_prefill_split_record_bytes.restype = c_long
@@ -1329,5 +1329,5 @@ from .latent import (add_rms_norm, build_latent_tiles, embed_scale, gate_up_glu_
                      latent_kv_write, latent_mfma_supported, latent_tile_kernel_takes, moe_finish, relu_sq, rms_norm_rows, rope_pairs, sigmoid_gate)
 
 # --------------------------------------------------------------------------- recurrent mixers, windowed attention, Dynamic Tanh
-from .seqmix import (add_dyt_norm, head_rms_norm, mix_heads, recurrent_scan, short_conv_qkv, up_xielu,  # noqa: E402,F401
-                     window_attention, window_cache_elems, xielu)
+from .seqmix import (add_dyt_norm, build_window_tiles, head_rms_norm, mix_heads, recurrent_scan, short_conv_qkv,  # noqa: E402,F401
+                     up_xielu, window_attention, window_cache_elems, window_mfma_supported, xielu)

@@ -534,10 +534,13 @@ def head_rms_norm(o, eps, weight, gate, out_dtype):
 
 
 def window_cache_views(pool, cache_off, kv_heads, dim, vdim):
-    """K [pages, PAGE, kv_heads, dim] and V [pages, PAGE, kv_heads, vdim] of one layer (views of the pool)."""
+    """K [pages, PAGE, kv_heads, dim] and V [pages, PAGE, kv_heads, vdim] of one layer: views of the pool
+    (indexed reads and writes go through).  In a page, K is stored key by key ([PAGE][kv_heads * dim]) and V
+    transposed ([kv_heads * vdim][PAGE]: a channel's 64 keys are contiguous, which is what the second matrix
+    product of the attention kernels reads)."""
     nk, nv = PAGE * kv_heads * dim, PAGE * kv_heads * vdim
     k = pool[:, cache_off:cache_off + nk].view(pool.shape[0], PAGE, kv_heads, dim)
-    v = pool[:, cache_off + nk:cache_off + nk + nv].view(pool.shape[0], PAGE, kv_heads, vdim)
+    v = pool[:, cache_off + nk:cache_off + nk + nv].view(pool.shape[0], kv_heads, vdim, PAGE).permute(0, 3, 1, 2)
     return k, v
 
 

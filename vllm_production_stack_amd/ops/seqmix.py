@@ -182,12 +182,43 @@ def short_conv_qkv(proj, conv_w, heads: int, kv_heads: int, dim: int, vdim: int,
     return q
 
 
+WINDOW_TILE_SLOTS = 64  # (row, query head) pairs of one tile of the matrix-core kernel
+WINDOW_MFMA = True      # False: every call takes the plain kernel (A/B runs, tests of the plain kernel)
+
+
+def window_mfma_supported(heads: int, kv_heads: int, dim: int, vdim: int) -> bool:
+    return bool(_ops()._kernels().vpsa_window_mfma_supported(c_int(heads), c_int(kv_heads), c_int(dim), c_int(vdim)))
+
+
+def build_window_tiles(q_lens, ctx_lens, heads: int, kv_heads: int):
+    """Work list of the matrix-core kernel for the prefill part of a batch: int32 rows (sequence, first
+    query row, rows, position of the first row); a tile holds consecutive rows of one sequence, as many as
+    fit 64 (row, query head of one KV group) pairs.  Latest rows first (they visit the most pages)."""
+    import numpy as np
+
+    per = max(1, WINDOW_TILE_SLOTS // (heads // kv_heads))
+    parts = []
+    row = 0
+    for i, (n, ctx) in enumerate(zip(q_lens, ctx_lens)):
+        k = np.arange(0, n, per, dtype=np.int64)
+        parts.append(np.stack([np.full_like(k, i), row + k, np.minimum(per, n - k), ctx - n + k], axis=1))
+        row += n
+    if not parts:
+        return np.zeros((0, 4), dtype=np.int32)
+    tiles = np.concatenate(parts)
+    return tiles[np.argsort(-tiles[:, 3], kind="stable")].astype(np.int32)
+
+
 def window_attention(q, pool, cache_off: int, kv_heads: int, vdim: int, block_tables, row_seq, positions, window: int,
-                     keep_first: int, scale: float, softcap: float, sink, out=None):
+                     keep_first: int, scale: float, softcap: float, sink, out=None, tiles=None):
     """Query rows q [T, heads, dim] over their sequences' cached keys: row i at position p sees key j when
     j <= p and (p - j < window or j < keep_first).  score = cap * tanh(q . k * scale / cap) (cap 0: none);
     softmax with ``sink`` [heads] (fp32) in the denominator.  Returns u fp32 [T, heads, kv_heads, vdim]:
-    each head's weights applied to the values of every KV head (``mix_heads`` picks and mixes)."""
+    each head's weights applied to the values of every KV head (``mix_heads`` picks and mixes).
+
+    bf16 rows of a shape the matrix-core kernel tiles take it: decode batches (``row_seq`` None) as they
+    are, prefill rows when ``tiles`` (the device copy of ``build_window_tiles``) describes them.
+    Everything else takes the plain kernel."""
     t, heads, dim = q.shape
     if out is None:
         out = torch.empty((t, heads, kv_heads, vdim), dtype=torch.float32, device=q.device)
@@ -199,13 +230,26 @@ def window_attention(q, pool, cache_off: int, kv_heads: int, vdim: int, block_ta
     o = _ops()
     _f32(sink, out)
     _i32(row_seq, positions)
-    assert q.stride(2) == 1 and q.stride(1) == dim and block_tables.dtype == torch.int32 and block_tables.stride(1) == 1
+    assert q.is_contiguous() and block_tables.dtype == torch.int32 and block_tables.stride(1) == 1
     assert heads % kv_heads == 0 and cache_off + window_cache_elems(kv_heads, dim, vdim) <= pool.shape[1]
+    esz = pool.element_size()
+    assert (cache_off * esz) % 16 == 0 and (pool.stride(0) * esz) % 16 == 0 and pool.data_ptr() % 16 == 0
+    dt = _dt(q, pool)
+    if (WINDOW_MFMA and dt == 0 and (tiles is not None or row_seq is None) and window_mfma_supported(heads, kv_heads, dim, vdim)
+            and q.data_ptr() % 16 == 0 and out.data_ptr() % 16 == 0):
+        if tiles is not None:
+            assert tiles.dtype == torch.int32 and tiles.is_contiguous() and tiles.shape[1] == 4
+        o._check(o._kernels().vpsa_window_attention_mfma(
+            o._p(q), c_long(q.stride(0)), _at(pool, cache_off), c_long(pool.stride(0)), o._p(block_tables),
+            c_int(block_tables.stride(0)), o._p(tiles), o._p(positions), o._p(sink), o._p(out),
+            c_int(tiles.shape[0] if tiles is not None else t), c_int(heads), c_int(kv_heads), c_int(dim), c_int(vdim),
+            c_int(window), c_int(keep_first), c_float(scale), c_float(softcap), o._stream()), "window_attention_mfma")
+        return out
     o._check(o._kernels().vpsa_window_attention(
         o._p(q), c_long(q.stride(0)), _at(pool, cache_off), c_long(pool.stride(0)), o._p(block_tables),
         c_int(block_tables.stride(0)), o._p(row_seq), o._p(positions), o._p(sink), o._p(out), c_int(t), c_int(heads),
         c_int(kv_heads), c_int(dim), c_int(vdim), c_int(window), c_int(keep_first), c_float(scale), c_float(softcap),
-        c_int(_dt(q, pool)), o._stream()), "window_attention")
+        c_int(dt), o._stream()), "window_attention")
     return out
 
 
