@@ -93,26 +93,41 @@ __global__ __launch_bounds__(256) void add_dyt_kernel(float* __restrict__ residu
 }
 
 // ---------------------------------------------------------------------------------
-// One workgroup = 256 / R state columns of one head of one sequence; a state column's `dim` rows are
-// spread over R neighbouring lanes, RPT rows each (row i = j * R + lane group), all in registers.
-// A block of up to TB tokens is prepared in LDS (rotation or gates, fp32), then walked token by token.
-template <typename T, int RPT, bool GATED>
+// The recurrence S <- a_t (.) S + k_t v_t^T, o_t = S^T q_t with the state in registers.  A thread holds a tile
+// of RPT rows x 4 columns of S; a column group's `dim` rows are spread over R neighbouring lanes (row
+// i = j * R + lane group), a workgroup covers 1024 / R columns of one head.  A block of up to TB tokens is
+// prepared in LDS (rotation or gates, fp32), then walked token by token.
+//
+// PHASE 0: whole sequences, from and to their state slots (decode rows, short chunks).
+// Long chunks are cut into pieces that run side by side (the recurrence is linear in S):
+// PHASE 1: a piece's end state from zero (no outputs) -> ws_state[piece];
+//          scan_propagate_kernel then walks a sequence's pieces, S <- A_piece (.) S + end state, leaves every
+//          piece's START state in ws_state and the sequence's end state in its slot;
+// PHASE 2: a piece's outputs from its start state.
+template <typename T, int RPT, bool GATED, int PHASE>
 __global__ __launch_bounds__(256) void recurrent_scan_kernel(
     const T* __restrict__ proj, long p_stride, int q_col, int k_col, int v_col, int heads, int dim, int vdim,
     float* __restrict__ state, long state_stride, const int* __restrict__ seq_cu, const int* __restrict__ seq_state,
     const int* __restrict__ positions, const float* __restrict__ decay, const float* __restrict__ cos_sin, int rot_dims,
     int layout, float k_scale, const float* __restrict__ gate_bias, const float* __restrict__ gate_lower,
-    float* __restrict__ out, int R, int TB) {
+    float* __restrict__ out, int R, int TB, const int* __restrict__ pieces, float* __restrict__ ws_state) {
   extern __shared__ float smem[];
-  const int seq = blockIdx.z, head = blockIdx.y;
+  const int head = blockIdx.y;
+  int seq, r0, r1;
+  if (PHASE == 0) {
+    seq = blockIdx.z, r0 = seq_cu[seq], r1 = seq_cu[seq + 1];
+  } else {
+    const int* pc = pieces + 3 * blockIdx.z;
+    seq = pc[0], r0 = pc[1], r1 = pc[1] + pc[2];
+  }
   const int slot = seq_state[seq];
-  const int r0 = seq_cu[seq], r1 = seq_cu[seq + 1];
-  const int dimp = R * RPT, cols = 256 / R;
+  const int dimp = R * RPT, cols = (256 / R) * 4;
+  const int tid = threadIdx.x, rg = tid % R, cb = tid / R;
+  const int col = blockIdx.x * cols + cb * 4;
   if (slot < 0) {  // rows of no sequence (a padded batch): their output is zero
-    for (int e = threadIdx.x; e < (r1 - r0) * cols; e += 256) {
-      const int c = blockIdx.x * cols + e % cols;
-      if (c < vdim) out[((long)(r0 + e / cols) * heads + head) * vdim + c] = 0.f;
-    }
+    if (PHASE != 1 && rg == 0)
+      for (int r = r0; r < r1; ++r)
+        for (int c = col; c < min(col + 4, vdim); ++c) out[((long)r * heads + head) * vdim + c] = 0.f;
     return;
   }
   if (r1 <= r0) return;
@@ -120,16 +135,27 @@ __global__ __launch_bounds__(256) void recurrent_scan_kernel(
   float* ks = qs + TB * dimp;
   float* as = ks + TB * dimp;                       // gates (GATED only)
   float* vs = GATED ? as + TB * dimp : as;
-  const int tid = threadIdx.x, rg = tid % R, cb = tid / R;
-  const int col = blockIdx.x * cols + cb;
-  const bool colok = col < vdim;
-  float* st = state + (long)slot * state_stride + (long)head * dim * vdim;
-  const bool fresh = positions[r0] == 0;
-  float S[RPT];
+  float* st = PHASE == 0 ? state + (long)slot * state_stride + (long)head * dim * vdim
+                         : ws_state + ((long)blockIdx.z * heads + head) * dim * vdim;
+  const bool vec = (vdim & 3) == 0 && (reinterpret_cast<uintptr_t>(st) & 15) == 0;  // whole, aligned float4 columns
+  const bool fresh = PHASE == 1 || (PHASE == 0 && positions[r0] == 0);
+  float S[RPT][4];
 #pragma unroll
   for (int j = 0; j < RPT; ++j) {
     const int i = j * R + rg;
-    S[j] = (!fresh && colok && i < dim) ? st[(long)i * vdim + col] : 0.f;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) S[j][c] = 0.f;
+    if (!fresh && i < dim) {
+      if (vec && col < vdim) {
+        const f32x4 v4 = *reinterpret_cast<const f32x4*>(st + (long)i * vdim + col);
+#pragma unroll
+        for (int c = 0; c < 4; ++c) S[j][c] = v4[c];
+      } else {
+#pragma unroll
+        for (int c = 0; c < 4; ++c)
+          if (col + c < vdim) S[j][c] = st[(long)i * vdim + col + c];
+      }
+    }
   }
   const float dec = GATED ? 0.f : decay[head];
   for (int rb = r0; rb < r1; rb += TB) {
@@ -150,7 +176,7 @@ __global__ __launch_bounds__(256) void recurrent_scan_kernel(
           k = 1.f - a;
         } else {
           const float* cs = cos_sin + (long)positions[row] * rot_dims;
-          q = rotated([&](int c) { return Cv<T>::ld(qp + c); }, i, cs, rot_dims, layout);
+          if (PHASE != 1) q = rotated([&](int c) { return Cv<T>::ld(qp + c); }, i, cs, rot_dims, layout);
           k = rotated([&](int c) { return Cv<T>::ld(kp + c); }, i, cs, rot_dims, layout) * k_scale;
         }
       }
@@ -165,28 +191,96 @@ __global__ __launch_bounds__(256) void recurrent_scan_kernel(
     }
     __syncthreads();
     for (int tt = 0; tt < nb; ++tt) {
-      const float v = vs[tt * cols + cb];
+      const f32x4 v = *reinterpret_cast<const f32x4*>(vs + tt * cols + cb * 4);
       const float* qr = qs + tt * dimp + rg;
       const float* kr = ks + tt * dimp + rg;
       const float* ar = as + tt * dimp + rg;
-      float acc = 0.f;
+      float acc[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int j = 0; j < RPT; ++j) {
-        const float kv = kr[j * R] * v;
-        S[j] = GATED ? fmaf(ar[j * R], S[j], kv) : fmaf(dec, S[j], kv);
-        acc = fmaf(S[j], qr[j * R], acc);
-      }
-      for (int off = R >> 1; off > 0; off >>= 1) acc += __shfl_xor(acc, off, 64);
-      if (rg == 0 && colok) out[((long)(rb + tt) * heads + head) * vdim + col] = acc;
-    }
-  }
-  if (colok) {
+        const float k = kr[j * R], a = GATED ? ar[j * R] : dec, q = PHASE == 1 ? 0.f : qr[j * R];
 #pragma unroll
-    for (int j = 0; j < RPT; ++j) {
-      const int i = j * R + rg;
-      if (i < dim) st[(long)i * vdim + col] = S[j];
+        for (int c = 0; c < 4; ++c) {
+          S[j][c] = fmaf(a, S[j][c], k * v[c]);
+          if (PHASE != 1) acc[c] = fmaf(S[j][c], q, acc[c]);
+        }
+      }
+      if (PHASE != 1) {
+        for (int off = R >> 1; off > 0; off >>= 1) {
+#pragma unroll
+          for (int c = 0; c < 4; ++c) acc[c] += __shfl_xor(acc[c], off, 64);
+        }
+        if (rg == 0) {
+          float* op = out + ((long)(rb + tt) * heads + head) * vdim + col;
+          if ((vdim & 3) == 0 && col < vdim) *reinterpret_cast<f32x4*>(op) = (f32x4){acc[0], acc[1], acc[2], acc[3]};
+          else
+            for (int c = 0; c < 4; ++c)
+              if (col + c < vdim) op[c] = acc[c];
+        }
+      }
     }
   }
+  if (PHASE == 2) return;
+#pragma unroll
+  for (int j = 0; j < RPT; ++j) {
+    const int i = j * R + rg;
+    if (i >= dim) continue;
+    if (vec && col < vdim) {
+      *reinterpret_cast<f32x4*>(st + (long)i * vdim + col) = (f32x4){S[j][0], S[j][1], S[j][2], S[j][3]};
+    } else {
+#pragma unroll
+      for (int c = 0; c < 4; ++c)
+        if (col + c < vdim) st[(long)i * vdim + col + c] = S[j][c];
+    }
+  }
+}
+
+// A piece's total decay per state row, prod_t a_t[i] -> ws_decay[piece][head][i].  One workgroup per (piece, head).
+template <typename T, bool GATED>
+__global__ __launch_bounds__(128) void scan_decay_kernel(const T* __restrict__ proj, long p_stride, int k_col, int heads,
+                                                         int dim, const float* __restrict__ decay,
+                                                         const float* __restrict__ gate_bias,
+                                                         const float* __restrict__ gate_lower,
+                                                         const int* __restrict__ pieces, float* __restrict__ ws_decay) {
+  const int piece = blockIdx.x, head = blockIdx.y;
+  const int r0 = pieces[3 * piece + 1], n = pieces[3 * piece + 2];
+  for (int i = threadIdx.x; i < dim; i += 128) {
+    float p = 1.f;
+    if (GATED) {
+      const float lo = gate_lower[head * dim + i], b = gate_bias[head * dim + i];
+      for (int r = r0; r < r0 + n; ++r)
+        p *= lo + (1.f - lo) * sigm(Cv<T>::ld(proj + (long)r * p_stride + k_col + head * dim + i) + b);
+    } else {
+      const float d = decay[head];
+      for (int r = 0; r < n; ++r) p *= d;
+    }
+    ws_decay[((long)piece * heads + head) * dim + i] = p;
+  }
+}
+
+// Walks a sequence's pieces in order: ws_state[piece] (the piece's end state from zero) becomes its START
+// state, and the sequence's slot gets the end state.  One thread per state element.
+__global__ __launch_bounds__(256) void scan_propagate_kernel(float* __restrict__ ws_state, const float* __restrict__ ws_decay,
+                                                             float* __restrict__ state, long state_stride,
+                                                             const int* __restrict__ seq_cu,
+                                                             const int* __restrict__ seq_state,
+                                                             const int* __restrict__ seq_pieces,
+                                                             const int* __restrict__ positions, int heads, int dim,
+                                                             int vdim) {
+  const int seq = blockIdx.z, head = blockIdx.y;
+  const int slot = seq_state[seq];
+  const int e = blockIdx.x * 256 + threadIdx.x;
+  if (slot < 0 || e >= dim * vdim || seq_cu[seq + 1] <= seq_cu[seq]) return;
+  const int i = e / vdim;
+  float* st = state + (long)slot * state_stride + (long)head * dim * vdim + e;
+  float S = positions[seq_cu[seq]] == 0 ? 0.f : *st;
+  for (int pc = seq_pieces[seq]; pc < seq_pieces[seq + 1]; ++pc) {
+    float* w = ws_state + ((long)pc * heads + head) * dim * vdim + e;
+    const float end = *w;
+    *w = S;
+    S = fmaf(ws_decay[((long)pc * heads + head) * dim + i], S, end);
+  }
+  *st = S;
 }
 
 // one wave per (row, head)
@@ -609,7 +703,7 @@ VPSA_EXPORT int vpsa_add_dyt(float* residual, const void* d1, long s1, float c1,
   return 0;
 }
 
-// Rows of the state a lane holds and lanes per state column for a head of `dim` rows.
+// Rows of the state a lane holds and lanes per column group for a head of `dim` rows.
 static void scan_shape(int dim, int* rpt, int* r) {
   for (int p = 8;; p <<= 1) {
     int lanes = 1;
@@ -618,35 +712,57 @@ static void scan_shape(int dim, int* rpt, int* r) {
   }
 }
 
+// pieces: nullptr = every sequence in one go (its rows from seq_cu); else int32 [n_pieces][3] = (sequence, first row,
+// rows) in sequence order, seq_pieces int32 [n_seqs + 1] = a sequence's first piece, and the workspaces
+// ws_state fp32 [n_pieces, heads, dim, vdim], ws_decay fp32 [n_pieces, heads, dim].
 VPSA_EXPORT int vpsa_recurrent_scan(const void* proj, long p_stride, int q_col, int k_col, int v_col, int heads, int dim,
                                     int vdim, float* state, long state_stride, const int* seq_cu, const int* seq_state,
                                     int n_seqs, const int* positions, const float* decay, const float* cos_sin,
                                     int rot_dims, int layout, float k_scale, const float* gate_bias,
-                                    const float* gate_lower, float* out, int gated, int dt, hipStream_t stream) {
+                                    const float* gate_lower, float* out, int gated, const int* pieces,
+                                    const int* seq_pieces, int n_pieces, float* ws_state, float* ws_decay, int dt,
+                                    hipStream_t stream) {
   if (n_seqs <= 0) return 0;
   int rpt, r;
   scan_shape(dim, &rpt, &r);
   if (r > 64) return 2;
-  const int dimp = r * rpt, cols = 256 / r;
+  const int dimp = r * rpt, cols = (256 / r) * 4;
   const int per_tok = (gated ? 3 : 2) * dimp + cols;
   int tb = (48 * 1024 / 4) / per_tok;
   if (tb > 16) tb = 16;
   if (tb < 1) return 3;
   const size_t lds = (size_t)tb * per_tok * sizeof(float);
-  dim3 grid((vdim + cols - 1) / cols, heads, n_seqs);
-#define SCAN(RPT, G)                                                                                                   \
-  recurrent_scan_kernel<T, RPT, G><<<grid, 256, lds, stream>>>((const T*)proj, p_stride, q_col, k_col, v_col, heads,   \
-                                                               dim, vdim, state, state_stride, seq_cu, seq_state,      \
-                                                               positions, decay, cos_sin, rot_dims, layout, k_scale,   \
-                                                               gate_bias, gate_lower, out, r, tb)
-#define SCAN_R(G)                                  \
-  if (rpt == 8) SCAN(8, G);                        \
-  else if (rpt == 16) SCAN(16, G);                 \
-  else SCAN(32, G);
-  if (gated) { SM_DISPATCH(dt, SCAN_R(true)); }
-  else { SM_DISPATCH(dt, SCAN_R(false)); }
+  const int col_blocks = (vdim + cols - 1) / cols;
+#define SCAN(RPT, G, PH, NZ)                                                                                           \
+  recurrent_scan_kernel<T, RPT, G, PH><<<dim3(col_blocks, heads, NZ), 256, lds, stream>>>(                             \
+      (const T*)proj, p_stride, q_col, k_col, v_col, heads, dim, vdim, state, state_stride, seq_cu, seq_state,        \
+      positions, decay, cos_sin, rot_dims, layout, k_scale, gate_bias, gate_lower, out, r, tb, pieces, ws_state)
+#define SCAN_R(G, PH, NZ)                          \
+  if (rpt == 8) SCAN(8, G, PH, NZ);                \
+  else if (rpt == 16) SCAN(16, G, PH, NZ);         \
+  else SCAN(32, G, PH, NZ);
+#define SCAN_G(PH, NZ)                             \
+  if (gated) { SCAN_R(true, PH, NZ) }              \
+  else { SCAN_R(false, PH, NZ) }
+  if (!pieces) {
+    SM_DISPATCH(dt, SCAN_G(0, n_seqs));
+    return 0;
+  }
+  if (n_pieces <= 0 || !seq_pieces || !ws_state || !ws_decay) return 4;
+  if (gated) {
+    SM_DISPATCH(dt, (scan_decay_kernel<T, true><<<dim3(n_pieces, heads), 128, 0, stream>>>(
+                        (const T*)proj, p_stride, k_col, heads, dim, decay, gate_bias, gate_lower, pieces, ws_decay)));
+  } else {
+    SM_DISPATCH(dt, (scan_decay_kernel<T, false><<<dim3(n_pieces, heads), 128, 0, stream>>>(
+                        (const T*)proj, p_stride, k_col, heads, dim, decay, gate_bias, gate_lower, pieces, ws_decay)));
+  }
+  SM_DISPATCH(dt, SCAN_G(1, n_pieces));
+  scan_propagate_kernel<<<dim3((dim * vdim + 255) / 256, heads, n_seqs), 256, 0, stream>>>(
+      ws_state, ws_decay, state, state_stride, seq_cu, seq_state, seq_pieces, positions, heads, dim, vdim);
+  SM_DISPATCH(dt, SCAN_G(2, n_pieces));
 #undef SCAN
 #undef SCAN_R
+#undef SCAN_G
   return 0;
 }
 

@@ -155,6 +155,39 @@ def case_recurrences(dev, dtype, tol):
             assert (out[:6] == 0).all() and torch.equal(torch.nan_to_num(state), torch.nan_to_num(before))
 
 
+def case_recurrence_pieces(dev, dtype, tol):
+    """Long chunks cut into pieces that run side by side: same outputs and same state as walking them in
+    one go, with a continued sequence, a new one and a one-row sequence in the same launch."""
+    dt = DTYPES[dtype]
+    g = torch.Generator().manual_seed(7)
+    for heads, dim, vdim in ((2, 16, 24), (2, 128, 64), (1, 40, 70)):
+        lens, starts, slots = [300, 1, 140], [77, 500, 0], [2, 0, 1]
+        t = sum(lens)
+        cols = (0, heads * dim, 2 * heads * dim)
+        proj = (torch.randn(t, heads * (2 * dim + vdim), generator=g) * 0.5).to(dt).to(dev)
+        decay = torch.tensor([1 - 2.0 ** -(3 + h) for h in range(heads)]).to(dev)
+        table = ops.build_cos_sin(dim, 1024, 500.0).to(dev)
+        bias, lower = torch.randn(heads * dim, generator=g).to(dev), (torch.rand(heads * dim, generator=g) * 0.9).to(dev)
+        pos, cu = [], [0]
+        for n, p0 in zip(lens, starts):
+            pos += list(range(p0, p0 + n))
+            cu.append(cu[-1] + n)
+        cut = ops.build_scan_pieces(lens, target=12)
+        assert cut is not None and cut[0].shape[0] > 5
+        pieces = tuple(torch.from_numpy(a).to(dev) for a in cut)
+        for kw in (dict(decay=decay, cos_sin=table, rot_dims=dim, layout=0, k_scale=dim ** -0.5),
+                   dict(gate_bias=bias, gate_lower=lower)):
+            s0 = torch.randn(3, heads * dim * vdim + 4, generator=g).to(dev)
+            res = []
+            for pc in (None, pieces):
+                state = s0.clone()
+                out = ops.recurrent_scan(proj, *cols, heads, dim, vdim, state, 4, i32(cu, dev), i32(slots, dev), i32(pos, dev),
+                                         pieces=pc, **kw)
+                res.append((out, state))
+            close(res[1][0], res[0][0].double().cpu(), tol, "outputs of the pieces")
+            close(res[1][1], res[0][1].double().cpu(), tol, "state after the pieces")
+
+
 def case_head_norm(dev, dtype, tol):
     dt = DTYPES[dtype]
     g = torch.Generator().manual_seed(2)

@@ -41,6 +41,11 @@ def test_recurrences(dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_recurrence_in_pieces(dtype):
+    rc.case_recurrence_pieces(DEV, dtype, 2e-5)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_head_norm(dtype):
     rc.case_head_norm(DEV, dtype, KERNEL_TOL[dtype])
 

@@ -52,4 +52,5 @@ class BatchMeta:
     seq_cu: torch.Tensor | None = None      # int32 [S + 1]: first row of every sequence
     seq_state: torch.Tensor | None = None   # int32 [S]: the sequence's state slot, -1 = rows of no sequence
     row_seq: torch.Tensor | None = None     # int32 [T]: the row's sequence (None: row i is sequence i)
+    scan_pieces: tuple | None = None        # long chunks cut into pieces for the recurrence kernels (ops.build_scan_pieces)
     pre_win_tiles: dict | None = None       # (heads, kv_heads) -> int32 [tiles, 4]: work lists of the windowed-attention tile kernel

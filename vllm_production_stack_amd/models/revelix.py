@@ -75,16 +75,21 @@ class RevelixModel:
         self.cache_offsets: dict[int, int] = {}
         self.state_offsets: dict[int, tuple] = {}
         c_off = s_off = 0
+
+        def up4(n):  # parts of a slot start on 16-byte boundaries (the kernels then move whole float4)
+            return (n + 3) // 4 * 4
+
         for i, s in enumerate(self.specs):
             m = s.mixer
             if isinstance(m, ParallelMixerSpec):
                 self.cache_offsets[i] = c_off
                 c_off += PAGE * m.left.cache_elems()
-                self.state_offsets[i] = (s_off, s_off + m.left.state_elems())
-                s_off += m.left.state_elems() + m.right.state_elems()
+                right = s_off + up4(m.left.state_elems())
+                self.state_offsets[i] = (s_off, right)
+                s_off = right + up4(m.right.state_elems())
             else:
                 self.state_offsets[i] = (s_off, None)
-                s_off += m.state_elems()
+                s_off += up4(m.state_elems())
         self.page_elems = max(c_off, 8)   # a model of recurrences only still names (empty) pages
         self.state_elems = max(s_off, 8)
         self._tables: dict[tuple, torch.Tensor] = {}
@@ -201,6 +206,9 @@ class RevelixModel:
         meta.seq_cu = to_dev(cu, torch.int32)
         meta.seq_state = to_dev(plan["state_slots"], torch.int32)
         meta.row_seq = to_dev(seq, torch.int32)
+        cut = ops.build_scan_pieces(q_lens) if self.device.type == "cuda" else None
+        if cut is not None:
+            meta.scan_pieces = tuple(torch.from_numpy(a).pin_memory().to(self.device, non_blocking=True) for a in cut)
         if plan["num_prefill"]:
             meta.pre_row_seq = to_dev([s - nd for s in seq[nd:]], torch.int32)
             meta.pre_win_tiles = {}
@@ -225,7 +233,7 @@ class RevelixModel:
         proj = ops.linear(h, lw.w_in)  # q | k | v | g
         o = ops.recurrent_scan(proj, 0, hd, 2 * hd, m.heads, m.dim, m.vdim, self.state, lw.state_off, meta.seq_cu,
                                meta.seq_state, meta.positions, decay=lw.decay, cos_sin=lw.cos_sin, rot_dims=m.rot.dims,
-                               layout=LAYOUTS[m.rot.layout], k_scale=m.dim ** -0.5)
+                               layout=LAYOUTS[m.rot.layout], k_scale=m.dim ** -0.5, pieces=meta.scan_pieces)
         y = ops.head_rms_norm(o, self.cfg.norm_eps, self.dtype, gate=proj[:, 2 * hd + hv:2 * hd + 2 * hv])
         return ops.linear(y, lw.w_o)
 
@@ -250,7 +258,7 @@ class RevelixModel:
         rd = r.heads * r.dim
         o = ops.recurrent_scan(proj, c0, c0 + rd, c0 + 2 * rd, r.heads, r.dim, r.vdim, self.state, lw.state_off_right,
                                meta.seq_cu, meta.seq_state, meta.positions, gate_bias=lw.gate_bias,
-                               gate_lower=lw.gate_lower)
+                               gate_lower=lw.gate_lower, pieces=meta.scan_pieces)
         right = ops.linear(ops.head_rms_norm(o, self.cfg.norm_eps, self.dtype, weight=lw.r_norm), lw.wr_o)
         return [(left, m.left_scale), (right, m.right_scale)]
 

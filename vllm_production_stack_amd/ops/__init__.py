@@ -1329,5 +1329,5 @@ from .latent import (add_rms_norm, build_latent_tiles, embed_scale, gate_up_glu_
                      latent_kv_write, latent_mfma_supported, latent_tile_kernel_takes, moe_finish, relu_sq, rms_norm_rows, rope_pairs, sigmoid_gate)
 
 # --------------------------------------------------------------------------- recurrent mixers, windowed attention, Dynamic Tanh
-from .seqmix import (add_dyt_norm, build_window_tiles, head_rms_norm, mix_heads, recurrent_scan, short_conv_qkv,  # noqa: E402,F401
+from .seqmix import (add_dyt_norm, build_scan_pieces, build_window_tiles, head_rms_norm, mix_heads, recurrent_scan, short_conv_qkv,  # noqa: E402,F401
                      up_xielu, window_attention, window_cache_elems, window_mfma_supported, xielu)

@@ -93,9 +93,32 @@ def add_dyt_norm(residual, deltas, weight, bias, alpha, out_dtype, want_out: boo
     return y
 
 
+SCAN_PIECE_MIN_ROWS = 128   # sequences of a step shorter than this are walked in one go
+SCAN_PIECES_TARGET = 48     # pieces per launch that fill the chip (times heads and column blocks)
+
+
+def build_scan_pieces(q_lens, target: int = SCAN_PIECES_TARGET):
+    """Cuts the sequences of a step into pieces the recurrence kernels run side by side.  Returns None when
+    no sequence is long enough to pay for it, else (pieces int32 [n, 3] = (sequence, first row, rows),
+    seq_pieces int32 [S + 1] = a sequence's first piece)."""
+    import numpy as np
+
+    if not q_lens or max(q_lens) < SCAN_PIECE_MIN_ROWS:
+        return None
+    total = sum(q_lens)
+    size = min(512, max(64, (total // target + 15) // 16 * 16))
+    pieces, first, row = [], [0], 0
+    for i, n in enumerate(q_lens):
+        for k in range(0, n, size):
+            pieces.append((i, row + k, min(size, n - k)))
+        row += n
+        first.append(len(pieces))
+    return np.asarray(pieces, dtype=np.int32).reshape(-1, 3), np.asarray(first, dtype=np.int32)
+
+
 def recurrent_scan(proj, q_col: int, k_col: int, v_col: int, heads: int, dim: int, vdim: int, state, state_off: int,
                    seq_cu, seq_state, positions, *, decay=None, cos_sin=None, rot_dims: int = 0, layout: int = 0,
-                   k_scale: float = 1.0, gate_bias=None, gate_lower=None):
+                   k_scale: float = 1.0, gate_bias=None, gate_lower=None, pieces=None):
     """Per sequence and head, over the sequence's rows in order: S <- a_t (.) S + k_t v_t^T, o_t = S^T q_t
     with S [dim, vdim] carried in the sequence's state slot.  q, k and v are column ranges of ``proj``
     [T, cols] (heads side by side).
@@ -106,6 +129,10 @@ def recurrent_scan(proj, q_col: int, k_col: int, v_col: int, heads: int, dim: in
 
     ``gate_bias`` / ``gate_lower`` (fp32 [heads * dim]) instead: the k columns hold gate logits,
     a_t = lower + (1 - lower) sigmoid(logit + bias) per row of S, k_t = 1 - a_t, q = silu(q).
+
+    ``pieces``: device copies of ``build_scan_pieces`` for steps with long chunks: the pieces' end states
+    from zero are computed side by side, chained per sequence (the recurrence is linear in S), and the
+    outputs of all pieces are computed side by side from their start states.
 
     Returns o fp32 [T, heads, vdim]."""
     gated = decay is None
@@ -121,12 +148,21 @@ def recurrent_scan(proj, q_col: int, k_col: int, v_col: int, heads: int, dim: in
     assert (gate_bias is not None and gate_lower is not None) if gated else (rot_dims == 0 or cos_sin.shape[1] == rot_dims)
     assert rot_dims <= dim and rot_dims % 2 == 0
     out = torch.empty((proj.shape[0], heads, vdim), dtype=torch.float32, device=proj.device)
+    pc = sp = ws_state = ws_decay = None
+    n_pieces = 0
+    if pieces is not None:
+        pc, sp = pieces
+        _i32(pc, sp)
+        n_pieces = pc.shape[0]
+        assert pc.shape[1] == 3 and sp.numel() == seq_cu.numel()
+        ws_state = torch.empty((n_pieces, heads, dim, vdim), dtype=torch.float32, device=proj.device)
+        ws_decay = torch.empty((n_pieces, heads, dim), dtype=torch.float32, device=proj.device)
     o._check(o._kernels().vpsa_recurrent_scan(
         o._p(proj), c_long(proj.stride(0)), c_int(q_col), c_int(k_col), c_int(v_col), c_int(heads), c_int(dim),
         c_int(vdim), _at(state, state_off), c_long(state.stride(0)), o._p(seq_cu), o._p(seq_state),
         c_int(seq_state.numel()), o._p(positions), o._p(decay), o._p(cos_sin), c_int(rot_dims), c_int(layout),
-        c_float(k_scale), o._p(gate_bias), o._p(gate_lower), o._p(out), c_int(1 if gated else 0), c_int(_dt(proj)),
-        o._stream()), "recurrent_scan")
+        c_float(k_scale), o._p(gate_bias), o._p(gate_lower), o._p(out), c_int(1 if gated else 0), o._p(pc), o._p(sp),
+        c_int(n_pieces), o._p(ws_state), o._p(ws_decay), c_int(_dt(proj)), o._stream()), "recurrent_scan")
     return out
 
 
