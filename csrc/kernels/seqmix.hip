@@ -19,6 +19,7 @@
 //
 // Plain kernels: every size is taken (bounds below are checked by the entry points).
 #include "common.h"
+#include <stdlib.h>
 
 namespace {
 
@@ -93,6 +94,42 @@ __global__ __launch_bounds__(256) void add_dyt_kernel(float* __restrict__ residu
 }
 
 // ---------------------------------------------------------------------------------
+// What enters a recurrence besides v, in fp32: prep [rows, heads, NP, dim] = q' | k' (| a).
+// Fixed decay (NP = 2): q and k rotated by the position's table row, k times k_scale.
+// Gated (NP = 3): q' = silu(q), a = lower + (1 - lower) sigmoid(logit + bias), k' = 1 - a.
+template <typename T, bool GATED>
+__global__ __launch_bounds__(256) void scan_prepare_kernel(const T* __restrict__ proj, long p_stride, int q_col, int k_col,
+                                                           int heads, int dim, const int* __restrict__ positions,
+                                                           const float* __restrict__ cos_sin, int rot_dims, int layout,
+                                                           float k_scale, const float* __restrict__ gate_bias,
+                                                           const float* __restrict__ gate_lower,
+                                                           float* __restrict__ prep) {
+  constexpr int NP = GATED ? 3 : 2;
+  const long row = blockIdx.x;
+  const T* qp = proj + row * p_stride + q_col;
+  const T* kp = proj + row * p_stride + k_col;
+  float* dst = prep + row * (long)heads * NP * dim;
+  const float* cs = GATED ? nullptr : cos_sin + (long)positions[row] * rot_dims;
+  for (int e = threadIdx.x; e < heads * dim; e += 256) {
+    const int h = e / dim, i = e - h * dim;
+    float* d = dst + (long)h * NP * dim + i;
+    if (GATED) {
+      const float x = Cv<T>::ld(qp + e);
+      const float lo = gate_lower[e];
+      const float a = lo + (1.f - lo) * sigm(Cv<T>::ld(kp + e) + gate_bias[e]);
+      d[0] = x * sigm(x);
+      d[dim] = 1.f - a;
+      d[2 * dim] = a;
+    } else {
+      const T* qh = qp + h * dim;
+      const T* kh = kp + h * dim;
+      d[0] = rotated([&](int c) { return Cv<T>::ld(qh + c); }, i, cs, rot_dims, layout);
+      d[dim] = rotated([&](int c) { return Cv<T>::ld(kh + c); }, i, cs, rot_dims, layout) * k_scale;
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------
 // The recurrence S <- a_t (.) S + k_t v_t^T, o_t = S^T q_t with the state in registers.  A thread holds a tile
 // of RPT rows x 4 columns of S; a column group's `dim` rows are spread over R neighbouring lanes (row
 // i = j * R + lane group), a workgroup covers 1024 / R columns of one head.  A block of up to TB tokens is
@@ -106,11 +143,11 @@ __global__ __launch_bounds__(256) void add_dyt_kernel(float* __restrict__ residu
 // PHASE 2: a piece's outputs from its start state.
 template <typename T, int RPT, bool GATED, int PHASE>
 __global__ __launch_bounds__(256) void recurrent_scan_kernel(
-    const T* __restrict__ proj, long p_stride, int q_col, int k_col, int v_col, int heads, int dim, int vdim,
+    const T* __restrict__ proj, long p_stride, int v_col, int heads, int dim, int vdim, const float* __restrict__ prep,
     float* __restrict__ state, long state_stride, const int* __restrict__ seq_cu, const int* __restrict__ seq_state,
-    const int* __restrict__ positions, const float* __restrict__ decay, const float* __restrict__ cos_sin, int rot_dims,
-    int layout, float k_scale, const float* __restrict__ gate_bias, const float* __restrict__ gate_lower,
-    float* __restrict__ out, int R, int TB, const int* __restrict__ pieces, float* __restrict__ ws_state) {
+    const int* __restrict__ positions, const float* __restrict__ decay, float* __restrict__ out, int R, int TB,
+    const int* __restrict__ pieces, float* __restrict__ ws_state) {
+  constexpr int NP = GATED ? 3 : 2;
   extern __shared__ float smem[];
   const int head = blockIdx.y;
   int seq, r0, r1;
@@ -142,7 +179,7 @@ __global__ __launch_bounds__(256) void recurrent_scan_kernel(
   float S[RPT][4];
 #pragma unroll
   for (int j = 0; j < RPT; ++j) {
-    const int i = j * R + rg;
+    const int i = ((j >> 2) * R + rg) * 4 + (j & 3);
 #pragma unroll
     for (int c = 0; c < 4; ++c) S[j][c] = 0.f;
     if (!fresh && i < dim) {
@@ -158,31 +195,17 @@ __global__ __launch_bounds__(256) void recurrent_scan_kernel(
     }
   }
   const float dec = GATED ? 0.f : decay[head];
+  if (dimp > dim)  // rows past the head's size stay zero in every staged block
+    for (int e = tid; e < TB * NP * dimp; e += 256) smem[e] = 0.f;
   for (int rb = r0; rb < r1; rb += TB) {
     const int nb = min(TB, r1 - rb);
     __syncthreads();
-    for (int e = tid; e < nb * dimp; e += 256) {
-      const int tt = e / dimp, i = e - tt * dimp;
-      const long row = rb + tt;
-      float q = 0.f, k = 0.f, a = 0.f;
-      if (i < dim) {
-        const T* qp = proj + row * p_stride + q_col + head * dim;
-        const T* kp = proj + row * p_stride + k_col + head * dim;
-        if (GATED) {
-          const float x = Cv<T>::ld(qp + i);
-          q = x * sigm(x);
-          const float lo = gate_lower[head * dim + i];
-          a = lo + (1.f - lo) * sigm(Cv<T>::ld(kp + i) + gate_bias[head * dim + i]);
-          k = 1.f - a;
-        } else {
-          const float* cs = cos_sin + (long)positions[row] * rot_dims;
-          if (PHASE != 1) q = rotated([&](int c) { return Cv<T>::ld(qp + c); }, i, cs, rot_dims, layout);
-          k = rotated([&](int c) { return Cv<T>::ld(kp + c); }, i, cs, rot_dims, layout) * k_scale;
-        }
-      }
-      qs[e] = q;
-      ks[e] = k;
-      if (GATED) as[e] = a;
+    for (int e = tid; e < nb * NP * dim; e += 256) {  // prepared rows are contiguous per (row, head)
+      const int tt = e / (NP * dim), rem = e - tt * (NP * dim);
+      const int which = rem / dim, i = rem - which * dim;
+      if (PHASE == 1 && which == 0) continue;         // no outputs: no queries
+      const float x = prep[((long)(rb + tt) * heads + head) * NP * dim + rem];
+      (which == 0 ? qs : which == 1 ? ks : as)[tt * dimp + i] = x;
     }
     for (int e = tid; e < nb * cols; e += 256) {
       const int tt = e / cols, c = e - tt * cols;
@@ -192,17 +215,24 @@ __global__ __launch_bounds__(256) void recurrent_scan_kernel(
     __syncthreads();
     for (int tt = 0; tt < nb; ++tt) {
       const f32x4 v = *reinterpret_cast<const f32x4*>(vs + tt * cols + cb * 4);
-      const float* qr = qs + tt * dimp + rg;
-      const float* kr = ks + tt * dimp + rg;
-      const float* ar = as + tt * dimp + rg;
+      const float* qr = qs + tt * dimp + rg * 4;
+      const float* kr = ks + tt * dimp + rg * 4;
+      const float* ar = as + tt * dimp + rg * 4;
       float acc[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int j = 0; j < RPT; ++j) {
-        const float k = kr[j * R], a = GATED ? ar[j * R] : dec, q = PHASE == 1 ? 0.f : qr[j * R];
+      for (int jg = 0; jg < RPT / 4; ++jg) {  // four rows per 16-byte LDS read
+        const f32x4 k4 = *reinterpret_cast<const f32x4*>(kr + jg * R * 4);
+        f32x4 q4 = {0.f, 0.f, 0.f, 0.f}, a4 = {dec, dec, dec, dec};
+        if (PHASE != 1) q4 = *reinterpret_cast<const f32x4*>(qr + jg * R * 4);
+        if (GATED) a4 = *reinterpret_cast<const f32x4*>(ar + jg * R * 4);
 #pragma unroll
-        for (int c = 0; c < 4; ++c) {
-          S[j][c] = fmaf(a, S[j][c], k * v[c]);
-          if (PHASE != 1) acc[c] = fmaf(S[j][c], q, acc[c]);
+        for (int jj = 0; jj < 4; ++jj) {
+          const int j = jg * 4 + jj;
+#pragma unroll
+          for (int c = 0; c < 4; ++c) {
+            S[j][c] = fmaf(a4[jj], S[j][c], k4[jj] * v[c]);
+            if (PHASE != 1) acc[c] = fmaf(S[j][c], q4[jj], acc[c]);
+          }
         }
       }
       if (PHASE != 1) {
@@ -223,7 +253,7 @@ __global__ __launch_bounds__(256) void recurrent_scan_kernel(
   if (PHASE == 2) return;
 #pragma unroll
   for (int j = 0; j < RPT; ++j) {
-    const int i = j * R + rg;
+    const int i = ((j >> 2) * R + rg) * 4 + (j & 3);
     if (i >= dim) continue;
     if (vec && col < vdim) {
       *reinterpret_cast<f32x4*>(st + (long)i * vdim + col) = (f32x4){S[j][0], S[j][1], S[j][2], S[j][3]};
@@ -703,26 +733,30 @@ VPSA_EXPORT int vpsa_add_dyt(float* residual, const void* d1, long s1, float c1,
   return 0;
 }
 
-// Rows of the state a lane holds and lanes per column group for a head of `dim` rows.
+// Rows of the state a lane holds and lanes per column group for a head of `dim` rows.  16 rows x 4 columns is the
+// largest tile that still leaves six waves per SIMD (128 x 256 states, 8192 rows: 1.25 ms against 2.3 ms with 32
+// rows and 1.4 ms with 8, which pays in cross-lane sums); heads beyond 1024 rows are refused.
 static void scan_shape(int dim, int* rpt, int* r) {
-  for (int p = 8;; p <<= 1) {
-    int lanes = 1;
-    while (lanes * p < dim) lanes <<= 1;
-    if (lanes <= 4 || p == 32) { *rpt = p; *r = lanes; return; }
-  }
+  static const int forced = getenv("VPSA_SCAN_ROWS") ? atoi(getenv("VPSA_SCAN_ROWS")) : 0;  // A/B runs: 8, 16 or 32
+  int p = (forced == 8 || forced == 16 || forced == 32) ? forced : (dim <= 32 ? 8 : 16);
+  int lanes = 1;
+  while (lanes * p < dim) lanes <<= 1;
+  *rpt = p;
+  *r = lanes;
 }
 
 // pieces: nullptr = every sequence in one go (its rows from seq_cu); else int32 [n_pieces][3] = (sequence, first row,
 // rows) in sequence order, seq_pieces int32 [n_seqs + 1] = a sequence's first piece, and the workspaces
-// ws_state fp32 [n_pieces, heads, dim, vdim], ws_decay fp32 [n_pieces, heads, dim].
+// ws_state fp32 [n_pieces, heads, dim, vdim], ws_decay fp32 [n_pieces, heads, dim].  prep: fp32 workspace
+// [rows, heads, 2 (3 when gated), dim].
 VPSA_EXPORT int vpsa_recurrent_scan(const void* proj, long p_stride, int q_col, int k_col, int v_col, int heads, int dim,
                                     int vdim, float* state, long state_stride, const int* seq_cu, const int* seq_state,
                                     int n_seqs, const int* positions, const float* decay, const float* cos_sin,
                                     int rot_dims, int layout, float k_scale, const float* gate_bias,
                                     const float* gate_lower, float* out, int gated, const int* pieces,
-                                    const int* seq_pieces, int n_pieces, float* ws_state, float* ws_decay, int dt,
-                                    hipStream_t stream) {
-  if (n_seqs <= 0) return 0;
+                                    const int* seq_pieces, int n_pieces, float* ws_state, float* ws_decay, float* prep,
+                                    int rows, int dt, hipStream_t stream) {
+  if (n_seqs <= 0 || rows <= 0) return 0;
   int rpt, r;
   scan_shape(dim, &rpt, &r);
   if (r > 64) return 2;
@@ -735,8 +769,8 @@ VPSA_EXPORT int vpsa_recurrent_scan(const void* proj, long p_stride, int q_col, 
   const int col_blocks = (vdim + cols - 1) / cols;
 #define SCAN(RPT, G, PH, NZ)                                                                                           \
   recurrent_scan_kernel<T, RPT, G, PH><<<dim3(col_blocks, heads, NZ), 256, lds, stream>>>(                             \
-      (const T*)proj, p_stride, q_col, k_col, v_col, heads, dim, vdim, state, state_stride, seq_cu, seq_state,        \
-      positions, decay, cos_sin, rot_dims, layout, k_scale, gate_bias, gate_lower, out, r, tb, pieces, ws_state)
+      (const T*)proj, p_stride, v_col, heads, dim, vdim, prep, state, state_stride, seq_cu, seq_state, positions,     \
+      decay, out, r, tb, pieces, ws_state)
 #define SCAN_R(G, PH, NZ)                          \
   if (rpt == 8) SCAN(8, G, PH, NZ);                \
   else if (rpt == 16) SCAN(16, G, PH, NZ);         \
@@ -744,6 +778,15 @@ VPSA_EXPORT int vpsa_recurrent_scan(const void* proj, long p_stride, int q_col, 
 #define SCAN_G(PH, NZ)                             \
   if (gated) { SCAN_R(true, PH, NZ) }              \
   else { SCAN_R(false, PH, NZ) }
+  if (gated) {
+    SM_DISPATCH(dt, (scan_prepare_kernel<T, true><<<rows, 256, 0, stream>>>((const T*)proj, p_stride, q_col, k_col, heads,
+                                                                            dim, positions, cos_sin, rot_dims, layout,
+                                                                            k_scale, gate_bias, gate_lower, prep)));
+  } else {
+    SM_DISPATCH(dt, (scan_prepare_kernel<T, false><<<rows, 256, 0, stream>>>((const T*)proj, p_stride, q_col, k_col, heads,
+                                                                             dim, positions, cos_sin, rot_dims, layout,
+                                                                             k_scale, gate_bias, gate_lower, prep)));
+  }
   if (!pieces) {
     SM_DISPATCH(dt, SCAN_G(0, n_seqs));
     return 0;

@@ -94,7 +94,7 @@ def add_dyt_norm(residual, deltas, weight, bias, alpha, out_dtype, want_out: boo
 
 
 SCAN_PIECE_MIN_ROWS = 128   # sequences of a step shorter than this are walked in one go
-SCAN_PIECES_TARGET = 48     # pieces per launch that fill the chip (times heads and column blocks)
+SCAN_PIECES_TARGET = 96     # pieces per launch that fill the chip (times heads and column blocks)
 
 
 def build_scan_pieces(q_lens, target: int = SCAN_PIECES_TARGET):
@@ -148,6 +148,8 @@ def recurrent_scan(proj, q_col: int, k_col: int, v_col: int, heads: int, dim: in
     assert (gate_bias is not None and gate_lower is not None) if gated else (rot_dims == 0 or cos_sin.shape[1] == rot_dims)
     assert rot_dims <= dim and rot_dims % 2 == 0
     out = torch.empty((proj.shape[0], heads, vdim), dtype=torch.float32, device=proj.device)
+    # what enters the recurrence besides v, prepared in fp32 by a pass of its own: q' | k' (| gates)
+    prep = torch.empty((proj.shape[0], heads, 3 if gated else 2, dim), dtype=torch.float32, device=proj.device)
     pc = sp = ws_state = ws_decay = None
     n_pieces = 0
     if pieces is not None:
@@ -162,7 +164,8 @@ def recurrent_scan(proj, q_col: int, k_col: int, v_col: int, heads: int, dim: in
         c_int(vdim), _at(state, state_off), c_long(state.stride(0)), o._p(seq_cu), o._p(seq_state),
         c_int(seq_state.numel()), o._p(positions), o._p(decay), o._p(cos_sin), c_int(rot_dims), c_int(layout),
         c_float(k_scale), o._p(gate_bias), o._p(gate_lower), o._p(out), c_int(1 if gated else 0), o._p(pc), o._p(sp),
-        c_int(n_pieces), o._p(ws_state), o._p(ws_decay), c_int(_dt(proj)), o._stream()), "recurrent_scan")
+        c_int(n_pieces), o._p(ws_state), o._p(ws_decay), o._p(prep), c_int(proj.shape[0]), c_int(_dt(proj)),
+        o._stream()), "recurrent_scan")
     return out
 
 
