@@ -537,7 +537,8 @@ __global__ __launch_bounds__(256) void window_mfma_kernel(
     const uint16_t* __restrict__ q, long q_stride, const uint16_t* __restrict__ cache, long page_stride,
     const int* __restrict__ block_tables, int bt_stride, const int* __restrict__ tiles,
     const int* __restrict__ positions, const float* __restrict__ sink, float* __restrict__ out, int heads, int kv_heads,
-    int window, int keep_first, float scale, float softcap) {
+    int window, int keep_first, float scale, float softcap, int splits, float* __restrict__ ws_o,
+    float* __restrict__ ws_ml) {
   constexpr int KS = DIM / 32;
   constexpr int DT = VALL / 16;
   constexpr int PK = DIM * 2 + 16;
@@ -577,8 +578,13 @@ __global__ __launch_bounds__(256) void window_mfma_kernel(
     if (valid) v = *reinterpret_cast<const u32x4*>(q + row * q_stride + (long)head * DIM + 32 * ks + 8 * g);
     qf[ks] = __builtin_bit_cast(bf16x8, v);
   }
-  float m = (sink && valid) ? sink[head] : -INFINITY;
-  float l = (sink && valid) ? 1.f : 0.f;
+  // key-range splits (decode rows in front of long windows): split blockIdx.z walks its share of the pages and
+  // leaves an unnormalised partial (o, max, sum); window_merge_kernel adds the sink and normalises
+  const int per = (walk.count + splits - 1) / splits;
+  const int i_begin = blockIdx.z * per, i_end = min(walk.count, i_begin + per);
+  const bool seeded = splits == 1 && sink && valid;
+  float m = seeded ? sink[head] : -INFINITY;
+  float l = seeded ? 1.f : 0.f;
   f32x4 o[DT];
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt) o[dt] = (f32x4){0.f, 0.f, 0.f, 0.f};
@@ -612,12 +618,12 @@ __global__ __launch_bounds__(256) void window_mfma_kernel(
   for (int nt = 0; nt < 4; ++nt) krow[nt] = (32 * (nt >> 1) + 8 * (c16 >> 2) + 4 * (nt & 1) + (c16 & 3)) * PK + 16 * g;
   const float inv_cap = softcap > 0.f ? 1.f / softcap : 0.f;
 
-  if (walk.count > 0) fetch(0);
-  for (int i = 0; i < walk.count; ++i) {
+  if (i_begin < i_end) fetch(i_begin);
+  for (int i = i_begin; i < i_end; ++i) {
     __syncthreads();  // the previous page's fragment reads are done
     stash();
     __syncthreads();
-    if (i + 1 < walk.count) fetch(i + 1);
+    if (i + 1 < i_end) fetch(i + 1);
     if (!wave_active) continue;
     const int j0 = walk.page(i) * PAGE;
     f32x4 s[4];
@@ -685,10 +691,45 @@ __global__ __launch_bounds__(256) void window_mfma_kernel(
       }
   }
   if (!valid) return;
-  const float inv = l > 0.f ? 1.f / l : 0.f;
-  float* dst = out + (row * heads + head) * (long)VALL + 4 * g;
+  if (splits == 1) {
+    const float inv = l > 0.f ? 1.f / l : 0.f;
+    float* dst = out + (row * heads + head) * (long)VALL + 4 * g;
 #pragma unroll
-  for (int dt = 0; dt < DT; ++dt) *reinterpret_cast<f32x4*>(dst + 16 * dt) = o[dt] * inv;
+    for (int dt = 0; dt < DT; ++dt) *reinterpret_cast<f32x4*>(dst + 16 * dt) = o[dt] * inv;
+  } else {
+    const long rec = (row * heads + head) * splits + blockIdx.z;
+    float* dst = ws_o + rec * VALL + 4 * g;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) *reinterpret_cast<f32x4*>(dst + 16 * dt) = o[dt];
+    if (g == 0) {
+      ws_ml[2 * rec] = m;
+      ws_ml[2 * rec + 1] = l;
+    }
+  }
+}
+
+// One workgroup per (row, head): out = sum_s o_s exp(m_s - M) / (sum_s l_s exp(m_s - M) + exp(sink - M))
+__global__ __launch_bounds__(128) void window_merge_kernel(const float* __restrict__ ws_o, const float* __restrict__ ws_ml,
+                                                           const float* __restrict__ sink, float* __restrict__ out,
+                                                           int heads, int vall, int splits) {
+  const long pair = blockIdx.x;
+  const int head = (int)(pair % heads);
+  float big = sink ? sink[head] : -INFINITY;
+  for (int s = 0; s < splits; ++s) big = fmaxf(big, ws_ml[2 * (pair * splits + s)]);
+  float den = sink ? __expf(sink[head] - big) : 0.f;
+  for (int s = 0; s < splits; ++s) {
+    const float ms = ws_ml[2 * (pair * splits + s)];
+    if (ms != -INFINITY) den += ws_ml[2 * (pair * splits + s) + 1] * __expf(ms - big);
+  }
+  const float inv = den > 0.f ? 1.f / den : 0.f;
+  for (int c = threadIdx.x; c < vall; c += 128) {
+    float acc = 0.f;
+    for (int s = 0; s < splits; ++s) {
+      const float ms = ws_ml[2 * (pair * splits + s)];
+      if (ms != -INFINITY) acc += ws_o[(pair * splits + s) * vall + c] * __expf(ms - big);
+    }
+    out[pair * vall + c] = acc * inv;
+  }
 }
 
 template <typename T>
@@ -861,7 +902,7 @@ template <int DIM, int VALL>
 static int launch_window_mfma(const void* q, long q_stride, const void* cache, long page_stride, const int* block_tables,
                               int bt_stride, const int* tiles, const int* positions, const float* sink, float* out,
                               int n_tiles, int heads, int kv_heads, int window, int keep_first, float scale,
-                              float softcap, hipStream_t st) {
+                              float softcap, int splits, float* ws_o, float* ws_ml, hipStream_t st) {
   constexpr int LDS = PAGE * (DIM * 2 + 16) + VALL * (PAGE * 2 + 16);
   static bool attr_set = false;
   if (!attr_set) {
@@ -870,9 +911,11 @@ static int launch_window_mfma(const void* q, long q_stride, const void* cache, l
       return -2;
     attr_set = true;
   }
-  window_mfma_kernel<DIM, VALL><<<dim3(n_tiles, kv_heads), dim3(256), LDS, st>>>(
+  window_mfma_kernel<DIM, VALL><<<dim3(n_tiles, kv_heads, splits), dim3(256), LDS, st>>>(
       (const uint16_t*)q, q_stride, (const uint16_t*)cache, page_stride, block_tables, bt_stride, tiles, positions, sink,
-      out, heads, kv_heads, window, keep_first, scale, softcap);
+      out, heads, kv_heads, window, keep_first, scale, softcap, splits, ws_o, ws_ml);
+  if (splits > 1)  // decode rows only: row r of the launch is row r of out
+    window_merge_kernel<<<n_tiles * heads, 128, 0, st>>>(ws_o, ws_ml, sink, out, heads, VALL, splits);
   return 0;
 }
 
@@ -882,14 +925,16 @@ VPSA_EXPORT int vpsa_window_attention_mfma(const void* q, long q_stride, const v
                                            const int* block_tables, int bt_stride, const int* tiles,
                                            const int* positions, const float* sink, float* out, int n_tiles, int heads,
                                            int kv_heads, int dim, int vdim, int window, int keep_first, float scale,
-                                           float softcap, hipStream_t stream) {
+                                           float softcap, int splits, float* ws_o, float* ws_ml, hipStream_t stream) {
   if (n_tiles <= 0) return 0;
   if (!vpsa_window_mfma_supported(heads, kv_heads, dim, vdim)) return 2;
+  if (splits < 1 || (splits > 1 && (tiles || !ws_o || !ws_ml))) return 3;  // splits are for decode rows
   const int vall = kv_heads * vdim;
 #define WM(D, V)                                                                                                      \
   if (dim == D && vall == V)                                                                                          \
     return launch_window_mfma<D, V>(q, q_stride, cache, page_stride, block_tables, bt_stride, tiles, positions, sink,  \
-                                    out, n_tiles, heads, kv_heads, window, keep_first, scale, softcap, stream);
+                                    out, n_tiles, heads, kv_heads, window, keep_first, scale, softcap, splits, ws_o,     \
+                                    ws_ml, stream);
   WM(64, 128) WM(64, 256) WM(64, 512) WM(128, 128) WM(128, 256) WM(128, 512)
 #undef WM
   return 2;

@@ -326,6 +326,11 @@ def case_window_tiles(dev, heads, kv_heads, dim, vdim, size, keep, tol=2e-2):
     u = ops.window_attention(q[rows].to(dev), pool, off, kv_heads, vdim, i32([order] * len(rows), dev), None,
                              i32([pos_q[r] for r in rows], dev), size, keep, scale, cap, sink.to(dev))
     close(ops.mix_heads(u, talk.to(dev), torch.float32).view(len(rows), heads, vdim), want[rows], tol, "decode rows")
+    for splits in (2, 3, 8):
+        u = ops.window_attention(q[rows].to(dev), pool, off, kv_heads, vdim, i32([order] * len(rows), dev), None,
+                                 i32([pos_q[r] for r in rows], dev), size, keep, scale, cap, sink.to(dev), splits=splits)
+        close(ops.mix_heads(u, talk.to(dev), torch.float32).view(len(rows), heads, vdim), want[rows], tol,
+              f"decode rows in {splits} key ranges")
 
 
 def case_short_conv(dev, dtype, tol):

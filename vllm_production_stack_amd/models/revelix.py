@@ -247,8 +247,13 @@ class RevelixModel:
         t, nd = h.shape[0], meta.num_decode
         u = torch.empty((t, a.heads, a.kv_heads, a.vdim), dtype=torch.float32, device=h.device)
         if nd > 0:
+            # the split count follows the batch rounded up to a power of two, which an eager step and the
+            # captured step of its batch bucket share: both then sum in the same order
+            splits = ops.window_decode_splits(1 << (nd - 1).bit_length(), a.kv_heads, a.window, a.keep_first,
+                                              self.max_model_len)
             ops.window_attention(q[:nd], pool, lw.cache_off, a.kv_heads, a.vdim, meta.dec_block_tables, None,
-                                 meta.positions[:nd], a.window, a.keep_first, a.scale, a.softcap, lw.sink, out=u[:nd])
+                                 meta.positions[:nd], a.window, a.keep_first, a.scale, a.softcap, lw.sink, out=u[:nd],
+                                 splits=splits)
         if meta.num_prefill_seqs > 0:
             ops.window_attention(q[nd:], pool, lw.cache_off, a.kv_heads, a.vdim, meta.pre_block_tables,
                                  meta.pre_row_seq, meta.positions[nd:], a.window, a.keep_first, a.scale, a.softcap,

@@ -1330,4 +1330,4 @@ from .latent import (add_rms_norm, build_latent_tiles, embed_scale, gate_up_glu_
 
 # --------------------------------------------------------------------------- recurrent mixers, windowed attention, Dynamic Tanh
 from .seqmix import (add_dyt_norm, build_scan_pieces, build_window_tiles, head_rms_norm, mix_heads, recurrent_scan, short_conv_qkv,  # noqa: E402,F401
-                     up_xielu, window_attention, window_cache_elems, window_mfma_supported, xielu)
+                     up_xielu, window_attention, window_cache_elems, window_decode_splits, window_mfma_supported, xielu)

@@ -248,16 +248,24 @@ def build_window_tiles(q_lens, ctx_lens, heads: int, kv_heads: int):
     return tiles[np.argsort(-tiles[:, 3], kind="stable")].astype(np.int32)
 
 
+def window_decode_splits(rows: int, kv_heads: int, window: int, keep_first: int, max_ctx: int) -> int:
+    """Key ranges per decode row: enough workgroups (rows x KV groups x splits) for about two per CU, none
+    shorter than two pages."""
+    pages = (min(window, max_ctx) + PAGE - 1) // PAGE + 1 + (keep_first + PAGE - 1) // PAGE
+    want = max(1, 512 // max(1, rows * kv_heads))
+    return max(1, min(want, pages // 2, 8))
+
+
 def window_attention(q, pool, cache_off: int, kv_heads: int, vdim: int, block_tables, row_seq, positions, window: int,
-                     keep_first: int, scale: float, softcap: float, sink, out=None, tiles=None):
+                     keep_first: int, scale: float, softcap: float, sink, out=None, tiles=None, splits: int = 1):
     """Query rows q [T, heads, dim] over their sequences' cached keys: row i at position p sees key j when
     j <= p and (p - j < window or j < keep_first).  score = cap * tanh(q . k * scale / cap) (cap 0: none);
     softmax with ``sink`` [heads] (fp32) in the denominator.  Returns u fp32 [T, heads, kv_heads, vdim]:
     each head's weights applied to the values of every KV head (``mix_heads`` picks and mixes).
 
     bf16 rows of a shape the matrix-core kernel tiles take it: decode batches (``row_seq`` None) as they
-    are, prefill rows when ``tiles`` (the device copy of ``build_window_tiles``) describes them.
-    Everything else takes the plain kernel."""
+    are (with ``splits`` key ranges per row, merged by a second launch), prefill rows when ``tiles`` (the
+    device copy of ``build_window_tiles``) describes them.  Everything else takes the plain kernel."""
     t, heads, dim = q.shape
     if out is None:
         out = torch.empty((t, heads, kv_heads, vdim), dtype=torch.float32, device=q.device)
@@ -276,13 +284,20 @@ def window_attention(q, pool, cache_off: int, kv_heads: int, vdim: int, block_ta
     dt = _dt(q, pool)
     if (WINDOW_MFMA and dt == 0 and (tiles is not None or row_seq is None) and window_mfma_supported(heads, kv_heads, dim, vdim)
             and q.data_ptr() % 16 == 0 and out.data_ptr() % 16 == 0):
+        ws_o = ws_ml = None
         if tiles is not None:
             assert tiles.dtype == torch.int32 and tiles.is_contiguous() and tiles.shape[1] == 4
+            splits = 1
+        elif splits > 1:
+            assert out.is_contiguous()
+            ws_o = torch.empty((t * heads * splits * kv_heads * vdim,), dtype=torch.float32, device=q.device)
+            ws_ml = torch.empty((t * heads * splits * 2,), dtype=torch.float32, device=q.device)
         o._check(o._kernels().vpsa_window_attention_mfma(
             o._p(q), c_long(q.stride(0)), _at(pool, cache_off), c_long(pool.stride(0)), o._p(block_tables),
             c_int(block_tables.stride(0)), o._p(tiles), o._p(positions), o._p(sink), o._p(out),
             c_int(tiles.shape[0] if tiles is not None else t), c_int(heads), c_int(kv_heads), c_int(dim), c_int(vdim),
-            c_int(window), c_int(keep_first), c_float(scale), c_float(softcap), o._stream()), "window_attention_mfma")
+            c_int(window), c_int(keep_first), c_float(scale), c_float(softcap), c_int(splits), o._p(ws_o), o._p(ws_ml),
+            o._stream()), "window_attention_mfma")
         return out
     o._check(o._kernels().vpsa_window_attention(
         o._p(q), c_long(q.stride(0)), _at(pool, cache_off), c_long(pool.stride(0)), o._p(block_tables),
