@@ -538,7 +538,7 @@ __global__ __launch_bounds__(256) void window_mfma_kernel(
     const int* __restrict__ block_tables, int bt_stride, const int* __restrict__ tiles,
     const int* __restrict__ positions, const float* __restrict__ sink, float* __restrict__ out, int heads, int kv_heads,
     int window, int keep_first, float scale, float softcap, int splits, float* __restrict__ ws_o,
-    float* __restrict__ ws_ml) {
+    float* __restrict__ ws_ml, int n_chunks) {
   constexpr int KS = DIM / 32;
   constexpr int DT = VALL / 16;
   constexpr int PK = DIM * 2 + 16;
@@ -550,7 +550,9 @@ __global__ __launch_bounds__(256) void window_mfma_kernel(
   char* vimg = lds + PAGE * PK;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int c16 = lane & 15, g = lane >> 4;
-  const int group = blockIdx.y, rep = heads / kv_heads;
+  // value channels beyond VALL are taken in chunks by workgroups of their own (each scores the keys again)
+  const int group = blockIdx.y / n_chunks, chunk = blockIdx.y % n_chunks, rep = heads / kv_heads;
+  const long vall_total = (long)n_chunks * VALL;
   int seq, row0, n_rows, pos0;
   if (tiles) {
     const int* e = tiles + 4 * blockIdx.x;
@@ -598,7 +600,8 @@ __global__ __launch_bounds__(256) void window_mfma_kernel(
       kb[b] = *reinterpret_cast<const u32x4*>(src + key * k_row + k_off + 8 * dc);
     }
 #pragma unroll
-    for (int b = 0; b < VB; ++b) vb[b] = *reinterpret_cast<const u32x4*>(src + v_off + (long)(tid + 256 * b) * 8);
+    for (int b = 0; b < VB; ++b)
+      vb[b] = *reinterpret_cast<const u32x4*>(src + v_off + (long)chunk * VALL * PAGE + (long)(tid + 256 * b) * 8);
   };
   auto stash = [&]() {
 #pragma unroll
@@ -693,15 +696,15 @@ __global__ __launch_bounds__(256) void window_mfma_kernel(
   if (!valid) return;
   if (splits == 1) {
     const float inv = l > 0.f ? 1.f / l : 0.f;
-    float* dst = out + (row * heads + head) * (long)VALL + 4 * g;
+    float* dst = out + (row * heads + head) * vall_total + (long)chunk * VALL + 4 * g;
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) *reinterpret_cast<f32x4*>(dst + 16 * dt) = o[dt] * inv;
   } else {
     const long rec = (row * heads + head) * splits + blockIdx.z;
-    float* dst = ws_o + rec * VALL + 4 * g;
+    float* dst = ws_o + rec * vall_total + (long)chunk * VALL + 4 * g;
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) *reinterpret_cast<f32x4*>(dst + 16 * dt) = o[dt];
-    if (g == 0) {
+    if (g == 0 && chunk == 0) {
       ws_ml[2 * rec] = m;
       ws_ml[2 * rec + 1] = l;
     }
@@ -732,12 +735,21 @@ __global__ __launch_bounds__(128) void window_merge_kernel(const float* __restri
   }
 }
 
-template <typename T>
+// One workgroup per row.  STAGED: the row's u [heads, kv_heads, vdim] goes through LDS in whole float4 (every
+// value is read by all the heads of its KV group); else every output reads its inputs from global memory.
+template <typename T, bool STAGED>
 __global__ __launch_bounds__(256) void mix_heads_kernel(const float* __restrict__ u, const float* __restrict__ talk,
                                                         T* __restrict__ y, int heads, int kv_heads, int vdim) {
+  extern __shared__ float us[];
   const long row = blockIdx.x;
   const int rep = heads / kv_heads;
-  const float* ur = u + row * (long)heads * kv_heads * vdim;
+  const int n = heads * kv_heads * vdim;
+  const float* ur = u + row * (long)n;
+  if (STAGED) {
+    for (int e = threadIdx.x * 4; e < n; e += 1024) *reinterpret_cast<f32x4*>(us + e) = *reinterpret_cast<const f32x4*>(ur + e);
+    __syncthreads();
+    ur = us;
+  }
   for (int e = threadIdx.x; e < heads * vdim; e += 256) {
     const int h = e / vdim, c = e - h * vdim;
     const int own = h / rep;
@@ -892,9 +904,15 @@ VPSA_EXPORT int vpsa_window_attention(const void* q, long q_stride, const void* 
   return 0;
 }
 
+// Value channels a workgroup of the matrix-core kernel takes (0: the shape is not tiled).
+static int window_chunk(int vall) {
+  for (int c = 512; c >= 128; c >>= 1)
+    if (vall % c == 0) return c;
+  return 0;
+}
+
 VPSA_EXPORT int vpsa_window_mfma_supported(int heads, int kv_heads, int dim, int vdim) {
-  const int vall = kv_heads * vdim;
-  return (dim == 64 || dim == 128) && (vall == 128 || vall == 256 || vall == 512) && heads % kv_heads == 0 &&
+  return (dim == 64 || dim == 128) && window_chunk(kv_heads * vdim) > 0 && heads % kv_heads == 0 &&
          heads / kv_heads <= 64;
 }
 
@@ -902,7 +920,7 @@ template <int DIM, int VALL>
 static int launch_window_mfma(const void* q, long q_stride, const void* cache, long page_stride, const int* block_tables,
                               int bt_stride, const int* tiles, const int* positions, const float* sink, float* out,
                               int n_tiles, int heads, int kv_heads, int window, int keep_first, float scale,
-                              float softcap, int splits, float* ws_o, float* ws_ml, hipStream_t st) {
+                              float softcap, int splits, float* ws_o, float* ws_ml, int n_chunks, hipStream_t st) {
   constexpr int LDS = PAGE * (DIM * 2 + 16) + VALL * (PAGE * 2 + 16);
   static bool attr_set = false;
   if (!attr_set) {
@@ -911,11 +929,11 @@ static int launch_window_mfma(const void* q, long q_stride, const void* cache, l
       return -2;
     attr_set = true;
   }
-  window_mfma_kernel<DIM, VALL><<<dim3(n_tiles, kv_heads, splits), dim3(256), LDS, st>>>(
+  window_mfma_kernel<DIM, VALL><<<dim3(n_tiles, kv_heads * n_chunks, splits), dim3(256), LDS, st>>>(
       (const uint16_t*)q, q_stride, (const uint16_t*)cache, page_stride, block_tables, bt_stride, tiles, positions, sink,
-      out, heads, kv_heads, window, keep_first, scale, softcap, splits, ws_o, ws_ml);
+      out, heads, kv_heads, window, keep_first, scale, softcap, splits, ws_o, ws_ml, n_chunks);
   if (splits > 1)  // decode rows only: row r of the launch is row r of out
-    window_merge_kernel<<<n_tiles * heads, 128, 0, st>>>(ws_o, ws_ml, sink, out, heads, VALL, splits);
+    window_merge_kernel<<<n_tiles * heads, 128, 0, st>>>(ws_o, ws_ml, sink, out, heads, VALL * n_chunks, splits);
   return 0;
 }
 
@@ -929,12 +947,12 @@ VPSA_EXPORT int vpsa_window_attention_mfma(const void* q, long q_stride, const v
   if (n_tiles <= 0) return 0;
   if (!vpsa_window_mfma_supported(heads, kv_heads, dim, vdim)) return 2;
   if (splits < 1 || (splits > 1 && (tiles || !ws_o || !ws_ml))) return 3;  // splits are for decode rows
-  const int vall = kv_heads * vdim;
+  const int vall = window_chunk(kv_heads * vdim), n_chunks = kv_heads * vdim / vall;
 #define WM(D, V)                                                                                                      \
   if (dim == D && vall == V)                                                                                          \
     return launch_window_mfma<D, V>(q, q_stride, cache, page_stride, block_tables, bt_stride, tiles, positions, sink,  \
                                     out, n_tiles, heads, kv_heads, window, keep_first, scale, softcap, splits, ws_o,     \
-                                    ws_ml, stream);
+                                    ws_ml, n_chunks, stream);
   WM(64, 128) WM(64, 256) WM(64, 512) WM(128, 128) WM(128, 256) WM(128, 512)
 #undef WM
   return 2;
@@ -943,7 +961,12 @@ VPSA_EXPORT int vpsa_window_attention_mfma(const void* q, long q_stride, const v
 VPSA_EXPORT int vpsa_mix_heads(const float* u, const float* talk, void* y, int rows, int heads, int kv_heads, int vdim,
                                int dt, hipStream_t stream) {
   if (rows <= 0) return 0;
-  SM_DISPATCH(dt, (mix_heads_kernel<T><<<rows, 256, 0, stream>>>(u, talk, (T*)y, heads, kv_heads, vdim)));
+  const size_t bytes = (size_t)heads * kv_heads * vdim * 4;
+  if (bytes <= 48 * 1024 && (heads * kv_heads * vdim) % 4 == 0 && ((uintptr_t)u & 15) == 0) {
+    SM_DISPATCH(dt, (mix_heads_kernel<T, true><<<rows, 256, bytes, stream>>>(u, talk, (T*)y, heads, kv_heads, vdim)));
+  } else {
+    SM_DISPATCH(dt, (mix_heads_kernel<T, false><<<rows, 256, 0, stream>>>(u, talk, (T*)y, heads, kv_heads, vdim)));
+  }
   return 0;
 }
 

@@ -56,6 +56,15 @@ def config_b():
     ], vocab=70, width=40, logit_scale=1.0, eps=1e-3)
 
 
+def config_c():
+    """Head sizes the matrix-core attention kernel tiles, and chunks long enough to be cut into pieces."""
+    return ro.make_config([
+        ro.retention_layer(heads=2, dim=64, vdim=64, rot_dims=32, mlp={"kind": "dense", "ff": 256}),
+        ro.parallel_layer(heads=4, kv_heads=2, dim=64, vdim=64, conv=4, size=100, keep=2, softcap=25.0, r_heads=2,
+                          r_dim=32, r_vdim=64, mlp={"kind": "dense", "ff": 256}),
+    ], vocab=200, width=128)
+
+
 # ----------------------------------------------------------------------------- mechanisms
 def case_dyt_and_xielu(dev, dtype, tol):
     dt = DTYPES[dtype]

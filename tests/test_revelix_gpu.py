@@ -63,7 +63,8 @@ def test_window_edges(dtype):
 
 @pytest.mark.parametrize("heads,kv_heads,dim,vdim,size,keep", [(4, 2, 64, 64, 70, 3), (8, 2, 128, 128, 100, 0),
                                                                 (3, 1, 64, 128, 64, 65), (16, 4, 128, 128, 129, 4),
-                                                                (4, 4, 128, 64, 1000, 2)])
+                                                                (4, 4, 128, 64, 1000, 2), (16, 8, 64, 128, 90, 5),
+                                                                (6, 3, 128, 128, 70, 1)])
 def test_window_attention_on_the_matrix_cores(heads, kv_heads, dim, vdim, size, keep):
     rc.case_window_tiles(DEV, heads, kv_heads, dim, vdim, size, keep)
 
@@ -84,6 +85,14 @@ def test_whole_decode_and_portions(dtype, tol, model_a):
 def test_other_sizes_and_first_tokens(dtype, tol, model_b):
     rc.check_cuts("cuda", dtype, tol, *model_b, 140, [[140], [1], [2, 1, 2], [3, 61, 64], [70, 5, 60]])
     rc.check_cuts("cuda", dtype, tol, *model_b, 3, [[3], [1, 2]])
+
+
+@pytest.mark.parametrize("dtype,tol", MODES)
+def test_tiled_attention_and_pieces_in_the_engine(dtype, tol):
+    cfg = rc.config_c()
+    w = ro.random_weights(cfg, seed=5)
+    assert ops.window_mfma_supported(4, 2, 64, 64) and ops.build_scan_pieces([300]) is not None
+    rc.check_cuts("cuda", dtype, tol, cfg, w, 300, [[300], [200, 100], [130, 1, 1, 168], [290]])
 
 
 @pytest.mark.parametrize("dtype,tol", MODES)

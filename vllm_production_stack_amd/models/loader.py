@@ -390,7 +390,7 @@ def _load_revelix(model: RevelixModel, ckpt_dir: Path) -> None:
                 if p.numel() != 2:
                     raise ValueError(f"{name}: two numbers expected")
                 sp = torch.nn.functional.softplus(p)
-                lw.act.copy_(torch.stack([sp[0], 0.5 + sp[1]]).float())
+                model.set_activation(lw, float(sp[0]), float(0.5 + sp[1]))
             else:
                 ok = False
         elif not isinstance(m, ParallelMixerSpec):

@@ -40,7 +40,7 @@ LAYOUTS = {"half": 0, "pairs": 1}
 
 class RevelixLayer:
     __slots__ = ("spec", "norm1", "norm2", "w_in", "b_in", "w_o", "decay", "cos_sin", "conv_w", "talk", "sink",
-                 "wr_o", "gate_bias", "gate_lower", "r_norm", "w_up", "w_down", "act", "cache_off", "state_off",
+                 "wr_o", "gate_bias", "gate_lower", "r_norm", "w_up", "w_down", "act", "act_host", "cache_off", "state_off",
                  "state_off_right")
 
     def __init__(self, spec):
@@ -167,9 +167,15 @@ class RevelixModel:
                 lw.norm2 = self._norm(g, w)
                 lw.w_up = self._alloc(g, f.ff, w)
                 lw.w_down = self._alloc(g, w, f.ff)
-                lw.act = torch.tensor([math.log(2.0), 0.5 + math.log(2.0)], dtype=f32, device=self.device)
+                self.set_activation(lw, math.log(2.0), 0.5 + math.log(2.0))
             self.layers.append(lw)
         self.norm = self._norm(g, w)
+
+    def set_activation(self, lw: RevelixLayer, a_pos: float, a_neg: float) -> None:
+        """The two curvatures of a layer's xIELU: on the device for the activation kernel (no host value
+        enters a captured step) and on the host for the GEMM epilogue's launch arguments."""
+        lw.act = torch.tensor([a_pos, a_neg], dtype=torch.float32, device=self.device)
+        lw.act_host = tuple(lw.act.tolist())
 
     @property
     def lm_head(self) -> torch.Tensor:  # the embedding table is the output matrix
@@ -279,7 +285,7 @@ class RevelixModel:
                 d = self._parallel(lw, h, pool, meta)
             if lw.spec.mlp is not None:
                 h = ops.add_dyt_norm(x, d, *lw.norm2, self.dtype)
-                d = [(ops.linear(ops.up_xielu(h, lw.w_up, lw.act), lw.w_down), 1.0)]
+                d = [(ops.linear(ops.up_xielu(h, lw.w_up, lw.act, lw.act_host), lw.w_down), 1.0)]
             if self.layer_probe is not None:
                 self.layer_probe(i, x + sum(t.float() * c for t, c in d))
         if meta.logits_rows is not None:

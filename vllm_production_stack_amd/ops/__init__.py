@@ -1190,7 +1190,7 @@ def tile_gemm_supported(n: int, k: int, silu_mul: bool = False) -> bool:
 
 
 def tile_gemm(a, w, offsets=None, rows=None, arow_idx=None, silu_mul=False, residual=None, out=None, glu_clamp=None,
-              relu_sq=False):
+              relu_sq=False, xielu=None):
     """The prefill GEMM (``csrc/kernels/tile_gemm.hip``): out[r] = epilogue(a[arow_idx[r] or r] @ w[g]^T).
 
     a [*, K] bf16; w [N, K] (dense) or [G, N, K] (grouped, with offsets [G + 1] int32 ON THE DEVICE:
@@ -1198,7 +1198,8 @@ def tile_gemm(a, w, offsets=None, rows=None, arow_idx=None, silu_mul=False, resi
     [gate rows | up rows], out = silu(gate) * up, [rows, N / 2].  residual [rows, N]: out = product +
     residual (``out`` may be ``residual`` itself).  glu_clamp = (limit, alpha, bias): w is [gate rows | up
     rows] as for silu_mul, out = min(g, limit) * sigmoid(alpha min(g, limit)) * (clamp(u, +-limit) + bias).
-    relu_sq: out = relu(product)^2.  Rows at or past offsets[G] are left unwritten."""
+    relu_sq: out = relu(product)^2.  xielu = (a_pos, a_neg): out = a_pos z^2 + z / 2 for z > 0, else
+    a_neg (exp(z) - 1 - z) + z / 2.  Rows at or past offsets[G] are left unwritten."""
     paired = silu_mul or glu_clamp is not None
     if w.dim() == 2:
         w = w.unsqueeze(0)
@@ -1208,7 +1209,7 @@ def tile_gemm(a, w, offsets=None, rows=None, arow_idx=None, silu_mul=False, resi
     n_out = n // 2 if paired else n
     _bf16_cuda(a, w, residual)
     assert w.is_contiguous() and a.stride(-1) == 1 and a.shape[1] == k
-    assert sum((silu_mul, glu_clamp is not None, relu_sq, residual is not None)) <= 1
+    assert sum((silu_mul, glu_clamp is not None, relu_sq, residual is not None, xielu is not None)) <= 1
     if offsets is not None:
         assert offsets.dtype == torch.int32 and offsets.numel() == g + 1 and offsets.is_cuda
     else:
@@ -1222,6 +1223,8 @@ def tile_gemm(a, w, offsets=None, rows=None, arow_idx=None, silu_mul=False, resi
         assert residual.stride(-1) == 1 and residual.shape[0] >= rows and residual.shape[1] == n_out
     epi = 1 if silu_mul else 2 if residual is not None else 3 if glu_clamp is not None else 4 if relu_sq else 0
     lim, alpha, bias = glu_clamp if glu_clamp is not None else (0.0, 1.0, 0.0)
+    if xielu is not None:
+        epi, alpha, bias = 5, float(xielu[0]), float(xielu[1])
     rc = _kernels().vpsa_tile_gemm(_p(a), c_long(a.stride(0)), _p(arow_idx), _p(w), _p(offsets), c_int(g), _p(out),
                                    c_long(out.stride(0)), c_int(rows), c_int(n), c_int(k), c_int(epi), _p(residual),
                                    c_long(residual.stride(0) if residual is not None else 0), c_long(a.shape[0]),

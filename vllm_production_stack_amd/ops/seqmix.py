@@ -336,6 +336,11 @@ def xielu(x, act):
     return y
 
 
-def up_xielu(x, w_up, act):
-    """xielu(x @ W.T)."""
-    return xielu(_ops().linear(x, w_up), act)
+def up_xielu(x, w_up, act, act_host=None):
+    """xielu(x @ W.T), in the prefill GEMM's epilogue when that kernel takes the shape (``act_host``: the two
+    numbers of ``act`` on the host, which the launch then carries as arguments)."""
+    o = _ops()
+    rows = o.tile_rows(x, w_up) if (x.is_cuda and act_host is not None) else 0
+    if rows:
+        return o.tile_gemm(x, w_up, xielu=act_host)
+    return xielu(o.linear(x, w_up), act)
