@@ -1,5 +1,5 @@
 // Sequence mixers with carried state, for gfx950: linear-attention recurrences (fixed decay per head, or a
-// forget gate per channel that also decides what is written), a short causal convolution in front of a
+// forget gate per channel whose complement is the write strength), a short causal convolution in front of a
 // windowed softmax attention with kept first tokens, capped scores, a sink and post-softmax head mixing,
 // the Dynamic Tanh norm on a 32-bit residual stream, and the xIELU activation.  bf16 or fp32 activations
 // (dtype 0 / 1 in the entry points); norms, angles, gates, decays, recurrent state, scores and softmax

@@ -15,7 +15,7 @@ F64 = torch.float64
 
 # ----------------------------------------------------------------------------- mechanisms
 def dyt(x, w, b, alpha):
-    """Dynamic Tanh: no mean, no variance."""
+    """Dynamic Tanh: an elementwise squashing norm without statistics."""
     return torch.tanh(alpha * x) * w + b
 
 
@@ -145,7 +145,7 @@ def window_attention(h, W, m: dict):
 
 
 def gated_recurrence(h, W, m: dict, eps: float):
-    """The right half of a 'parallel' mixer: the forget gate also decides what is written."""
+    """The right half of a 'parallel' mixer: input gate tied to the forget gate (1 - f is written where f is kept)."""
     t = h.shape[0]
     H, d, vd = int(m["heads"]), int(m["dim"]), int(m["vdim"])
     q = torch.nn.functional.silu(h @ W["q"].T).view(t, H, d)

@@ -92,7 +92,7 @@ class RotarySpec:
 
 @dataclass(frozen=True)
 class RetentionSpec:
-    """Linear attention with one fixed decay per head, no softmax and no denominator: per head a
+    """Un-normalised linear attention, one constant decay for each head: per head a
     ``dim`` x ``vdim`` state S <- decay S + k v^T, read by the rotated query; head outputs are brought
     to unit root mean square and gated by silu(W_g h)."""
     heads: int
@@ -144,7 +144,7 @@ class WindowAttentionSpec:
 
 @dataclass(frozen=True)
 class GatedRecurrenceSpec:
-    """Linear attention whose forget gate also decides what is written: S <- diag(f) S + (1 - f) v^T,
+    """Linear attention with the input gate tied to the forget gate: S <- diag(f) S + (1 - f) v^T,
     f = lower + (1 - lower) sigmoid(W_f h + b) per head and query channel; q = silu(W_q h); head
     outputs are RMS-normed with one weight vector shared by the heads."""
     heads: int

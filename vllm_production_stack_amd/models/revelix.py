@@ -8,12 +8,12 @@ feed-forward with the xIELU activation:
   projection; the recurrence kernel rotates q and k (pairs (i, i + dims / 2)), scales k, walks the
   chunk from the sequence's fp32 state slot and leaves the new state there; head outputs are brought to
   unit root mean square, gated by silu(g) and projected.
-- ``parallel``: two mixers side by side on the same input, one fused input projection
+- ``parallel``: a pair of mixers fed by the same normed input through one fused input projection
   (left q | k | v with biases, right q | gate logits | v).  Left: a short causal convolution on
   every q / k / v channel (its last rows per sequence live in the state slot), rotary positions with
   ramped frequency scaling, k and v into the paged pool, softmax attention over a sliding window that
   keeps the first tokens, with capped scores, a sink logit and the heads' weights mixed after the
-  softmax.  Right: linear attention whose forget gate also decides what is written, RMS-normed per
+  softmax.  Right: linear attention with the input gate tied to the forget gate, RMS-normed per
   head.  The layer adds ``left_scale * left + right_scale * right`` to the stream.
 
 Only windowed attention owns pool pages (K and V of every such layer, layer after layer inside a
