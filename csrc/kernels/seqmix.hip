@@ -735,27 +735,42 @@ __global__ __launch_bounds__(128) void window_merge_kernel(const float* __restri
   }
 }
 
-// One workgroup per row.  STAGED: the row's u [heads, kv_heads, vdim] goes through LDS in whole float4 (every
-// value is read by all the heads of its KV group); else every output reads its inputs from global memory.
+// One workgroup per row.  STAGED: KV head by KV head, the weighted values of every query head on that KV head
+// (u[:, kv, :], heads x vdim floats) go through LDS in whole float4, since every one of them is read by all the
+// heads of the group; else every output reads its inputs from global memory.
 template <typename T, bool STAGED>
 __global__ __launch_bounds__(256) void mix_heads_kernel(const float* __restrict__ u, const float* __restrict__ talk,
                                                         T* __restrict__ y, int heads, int kv_heads, int vdim) {
   extern __shared__ float us[];
   const long row = blockIdx.x;
   const int rep = heads / kv_heads;
-  const int n = heads * kv_heads * vdim;
-  const float* ur = u + row * (long)n;
-  if (STAGED) {
-    for (int e = threadIdx.x * 4; e < n; e += 1024) *reinterpret_cast<f32x4*>(us + e) = *reinterpret_cast<const f32x4*>(ur + e);
-    __syncthreads();
-    ur = us;
+  const float* ur = u + row * (long)heads * kv_heads * vdim;
+  T* yr = y + row * (long)heads * vdim;
+  if (!STAGED) {
+    for (int e = threadIdx.x; e < heads * vdim; e += 256) {
+      const int h = e / vdim, c = e - h * vdim;
+      const int own = h / rep;
+      float acc = 0.f;
+      for (int g = 0; g < heads; ++g) acc = fmaf(talk[h * heads + g], ur[((long)g * kv_heads + own) * vdim + c], acc);
+      Cv<T>::st(yr + e, acc);
+    }
+    return;
   }
-  for (int e = threadIdx.x; e < heads * vdim; e += 256) {
-    const int h = e / vdim, c = e - h * vdim;
-    const int own = h / rep;
-    float acc = 0.f;
-    for (int g = 0; g < heads; ++g) acc = fmaf(talk[h * heads + g], ur[((long)g * kv_heads + own) * vdim + c], acc);
-    Cv<T>::st(y + row * (long)heads * vdim + e, acc);
+  const int quads = vdim >> 2;
+  for (int own = 0; own < kv_heads; ++own) {
+    __syncthreads();
+    for (int e = threadIdx.x; e < heads * quads; e += 256) {
+      const int g = e / quads, c4 = e - g * quads;
+      *reinterpret_cast<f32x4*>(us + g * vdim + 4 * c4) =
+          *reinterpret_cast<const f32x4*>(ur + ((long)g * kv_heads + own) * vdim + 4 * c4);
+    }
+    __syncthreads();
+    for (int e = threadIdx.x; e < rep * vdim; e += 256) {
+      const int h = own * rep + e / vdim, c = e % vdim;
+      float acc = 0.f;
+      for (int g = 0; g < heads; ++g) acc = fmaf(talk[h * heads + g], us[g * vdim + c], acc);
+      Cv<T>::st(yr + (long)h * vdim + c, acc);
+    }
   }
 }
 
@@ -961,8 +976,8 @@ VPSA_EXPORT int vpsa_window_attention_mfma(const void* q, long q_stride, const v
 VPSA_EXPORT int vpsa_mix_heads(const float* u, const float* talk, void* y, int rows, int heads, int kv_heads, int vdim,
                                int dt, hipStream_t stream) {
   if (rows <= 0) return 0;
-  const size_t bytes = (size_t)heads * kv_heads * vdim * 4;
-  if (bytes <= 48 * 1024 && (heads * kv_heads * vdim) % 4 == 0 && ((uintptr_t)u & 15) == 0) {
+  const size_t bytes = (size_t)heads * vdim * 4;
+  if (bytes <= 48 * 1024 && vdim % 4 == 0 && ((uintptr_t)u & 15) == 0) {
     SM_DISPATCH(dt, (mix_heads_kernel<T, true><<<rows, 256, bytes, stream>>>(u, talk, (T*)y, heads, kv_heads, vdim)));
   } else {
     SM_DISPATCH(dt, (mix_heads_kernel<T, false><<<rows, 256, 0, stream>>>(u, talk, (T*)y, heads, kv_heads, vdim)));

@@ -76,6 +76,11 @@ def test_other_sizes_and_first_tokens(model_b):
     rc.check_cuts("cpu", "float32", TOL, *model_b, 3, [[3], [1, 2]])
 
 
+def test_one_kind_of_layer_only():
+    for cfg in (rc.config_d(), rc.config_e()):
+        rc.check_cuts("cpu", "float32", TOL, cfg, ro.random_weights(cfg, seed=6), 130, [[130], [66, 2, 1, 61], [1, 1, 1, 1, 3]])
+
+
 def test_long_decode(model_b):
     rc.check_cuts("cpu", "float32", TOL, *model_b, 330, [[20]], pages=6)  # 310 single tokens over five pages
 

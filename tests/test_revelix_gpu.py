@@ -96,6 +96,14 @@ def test_tiled_attention_and_pieces_in_the_engine(dtype, tol):
 
 
 @pytest.mark.parametrize("dtype,tol", MODES)
+def test_one_kind_of_layer_only(dtype, tol):
+    # widths of 16 and 24 average bf16 rounding over few terms: fp32 is the sharp run, bf16 a sanity bound
+    tol = tol if dtype == "float32" else 0.15
+    for cfg in (rc.config_d(), rc.config_e()):
+        rc.check_cuts("cuda", dtype, tol, cfg, ro.random_weights(cfg, seed=6), 130, [[130], [66, 2, 1, 61], [1, 1, 1, 1, 3]])
+
+
+@pytest.mark.parametrize("dtype,tol", MODES)
 def test_long_decode(dtype, tol, model_b):
     rc.check_cuts("cuda", dtype, tol, *model_b, 330, [[20]], pages=6)
 
