@@ -532,7 +532,7 @@ __global__ __launch_bounds__(256) void window_attention_kernel(
 // probabilities go from the first product's accumulators into the second without leaving the lane.
 // Scores are capped, masked by window / kept first tokens and normalised online in fp32; a sink logit starts
 // the running state (max = sink, sum = 1).  The next page's loads are in flight while a page is multiplied.
-template <int DIM, int VALL>
+template <int DIM, int VALL, int NSUB>
 __global__ __launch_bounds__(256) void window_mfma_kernel(
     const uint16_t* __restrict__ q, long q_stride, const uint16_t* __restrict__ cache, long page_stride,
     const int* __restrict__ block_tables, int bt_stride, const int* __restrict__ tiles,
@@ -561,35 +561,46 @@ __global__ __launch_bounds__(256) void window_mfma_kernel(
     seq = row0 = blockIdx.x, n_rows = 1, pos0 = positions[blockIdx.x];
   }
   if (seq < 0) return;
+  // a wave owns NSUB runs of 16 slots: every K and V^T fragment it reads from LDS serves all of them
   const int n_slots = n_rows * rep;
-  const int slot = wave * 16 + c16;
-  const bool valid = slot < n_slots;
-  const bool wave_active = wave * 16 < n_slots;  // wave-uniform
-  const int tok = valid ? slot / rep : 0;
-  const int head = group * rep + (valid ? slot % rep : 0);
-  const long row = row0 + tok;
-  const int my_pos = valid ? pos0 + tok : -1;
+  bool valid[NSUB];
+  int head[NSUB], my_pos[NSUB];
+  long row[NSUB];
+#pragma unroll
+  for (int u = 0; u < NSUB; ++u) {
+    const int slot = (wave * NSUB + u) * 16 + c16;
+    valid[u] = slot < n_slots;
+    const int tok = valid[u] ? slot / rep : 0;
+    head[u] = group * rep + (valid[u] ? slot % rep : 0);
+    row[u] = row0 + tok;
+    my_pos[u] = valid[u] ? pos0 + tok : -1;
+  }
+  const bool wave_active = wave * NSUB * 16 < n_slots;  // wave-uniform
   const PageWalk walk(pos0, pos0 + n_rows - 1, window, keep_first);
   const int* bt = block_tables + (long)seq * bt_stride;
   const long k_off = (long)group * DIM, k_row = (long)kv_heads * DIM, v_off = (long)PAGE * kv_heads * DIM;
 
-  bf16x8 qf[KS];
-#pragma unroll
-  for (int ks = 0; ks < KS; ++ks) {
-    u32x4 v = {0u, 0u, 0u, 0u};
-    if (valid) v = *reinterpret_cast<const u32x4*>(q + row * q_stride + (long)head * DIM + 32 * ks + 8 * g);
-    qf[ks] = __builtin_bit_cast(bf16x8, v);
-  }
+  bf16x8 qf[NSUB][KS];
+  float m[NSUB], l[NSUB];
+  f32x4 o[NSUB][DT];
   // key-range splits (decode rows in front of long windows): split blockIdx.z walks its share of the pages and
   // leaves an unnormalised partial (o, max, sum); window_merge_kernel adds the sink and normalises
   const int per = (walk.count + splits - 1) / splits;
   const int i_begin = blockIdx.z * per, i_end = min(walk.count, i_begin + per);
-  const bool seeded = splits == 1 && sink && valid;
-  float m = seeded ? sink[head] : -INFINITY;
-  float l = seeded ? 1.f : 0.f;
-  f32x4 o[DT];
 #pragma unroll
-  for (int dt = 0; dt < DT; ++dt) o[dt] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  for (int u = 0; u < NSUB; ++u) {
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      u32x4 v = {0u, 0u, 0u, 0u};
+      if (valid[u]) v = *reinterpret_cast<const u32x4*>(q + row[u] * q_stride + (long)head[u] * DIM + 32 * ks + 8 * g);
+      qf[u][ks] = __builtin_bit_cast(bf16x8, v);
+    }
+    const bool seeded = splits == 1 && sink && valid[u];
+    m[u] = seeded ? sink[head[u]] : -INFINITY;
+    l[u] = seeded ? 1.f : 0.f;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) o[u][dt] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  }
 
   u32x4 kb[KB], vb[VB];
   auto fetch = [&](int i) {
@@ -629,84 +640,100 @@ __global__ __launch_bounds__(256) void window_mfma_kernel(
     if (i + 1 < i_end) fetch(i + 1);
     if (!wave_active) continue;
     const int j0 = walk.page(i) * PAGE;
-    f32x4 s[4];
+    f32x4 s[NSUB][4];
 #pragma unroll
-    for (int nt = 0; nt < 4; ++nt) s[nt] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    for (int u = 0; u < NSUB; ++u)
+#pragma unroll
+      for (int nt = 0; nt < 4; ++nt) s[u][nt] = (f32x4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks)
 #pragma unroll
       for (int nt = 0; nt < 4; ++nt) {
         const bf16x8 a = *reinterpret_cast<const bf16x8*>(kimg + krow[nt] + 64 * ks);
-        s[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qf[ks], s[nt], 0, 0, 0);
+#pragma unroll
+        for (int u = 0; u < NSUB; ++u) s[u][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qf[u][ks], s[u][nt], 0, 0, 0);
       }
-    float mx = -INFINITY;
+    bf16x8 pf[NSUB][2];
+    bool rescale = false;
+    float corr[NSUB];
 #pragma unroll
-    for (int nt = 0; nt < 4; ++nt)
+    for (int u = 0; u < NSUB; ++u) {
+      float mx = -INFINITY;
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const int j = j0 + 32 * (nt >> 1) + 8 * g + 4 * (nt & 1) + e;
-        float v = -INFINITY;
-        if (key_seen(j, my_pos, window, keep_first)) {
-          v = s[nt][e] * scale;
-          if (softcap > 0.f) {  // cap * tanh(v / cap), tanh(x) = 1 - 2 / (exp(2 x) + 1)
-            const float x = v * inv_cap;
-            v = softcap * (1.f - 2.f / (__expf(2.f * x) + 1.f));
+      for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int j = j0 + 32 * (nt >> 1) + 8 * g + 4 * (nt & 1) + e;
+          float v = -INFINITY;
+          if (key_seen(j, my_pos[u], window, keep_first)) {
+            v = s[u][nt][e] * scale;
+            if (softcap > 0.f) {  // cap * tanh(v / cap), tanh(x) = 1 - 2 / (exp(2 x) + 1)
+              const float x = v * inv_cap;
+              v = softcap * (1.f - 2.f / (__expf(2.f * x) + 1.f));
+            }
           }
+          s[u][nt][e] = v;
+          mx = fmaxf(mx, v);
         }
-        s[nt][e] = v;
-        mx = fmaxf(mx, v);
+      mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      const float mn = fmaxf(m[u], mx);
+      const bool dead = mn == -INFINITY;
+      corr[u] = (dead || m[u] == -INFINITY) ? (dead ? 1.f : 0.f) : __expf(m[u] - mn);
+      float psum = 0.f;
+#pragma unroll
+      for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const float pv = dead ? 0.f : __expf(s[u][nt][e] - mn);
+          s[u][nt][e] = pv;
+          psum += pv;
+        }
+      psum += __shfl_xor(psum, 16, 64);
+      psum += __shfl_xor(psum, 32, 64);
+      l[u] = l[u] * corr[u] + psum;
+      m[u] = mn;
+#pragma unroll
+      for (int kk = 0; kk < 2; ++kk) {
+        u32x4 w = {pack_bf16x2(s[u][2 * kk][0], s[u][2 * kk][1]), pack_bf16x2(s[u][2 * kk][2], s[u][2 * kk][3]),
+                   pack_bf16x2(s[u][2 * kk + 1][0], s[u][2 * kk + 1][1]),
+                   pack_bf16x2(s[u][2 * kk + 1][2], s[u][2 * kk + 1][3])};
+        pf[u][kk] = __builtin_bit_cast(bf16x8, w);
       }
-    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-    const float mn = fmaxf(m, mx);
-    const bool dead = mn == -INFINITY;
-    const float corr = (dead || m == -INFINITY) ? (dead ? 1.f : 0.f) : __expf(m - mn);
-    float psum = 0.f;
-#pragma unroll
-    for (int nt = 0; nt < 4; ++nt)
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const float pv = dead ? 0.f : __expf(s[nt][e] - mn);
-        s[nt][e] = pv;
-        psum += pv;
-      }
-    psum += __shfl_xor(psum, 16, 64);
-    psum += __shfl_xor(psum, 32, 64);
-    l = l * corr + psum;
-    m = mn;
-    bf16x8 pf[2];
-#pragma unroll
-    for (int kk = 0; kk < 2; ++kk) {
-      u32x4 w = {pack_bf16x2(s[2 * kk][0], s[2 * kk][1]), pack_bf16x2(s[2 * kk][2], s[2 * kk][3]),
-                 pack_bf16x2(s[2 * kk + 1][0], s[2 * kk + 1][1]), pack_bf16x2(s[2 * kk + 1][2], s[2 * kk + 1][3])};
-      pf[kk] = __builtin_bit_cast(bf16x8, w);
+      rescale = rescale || !__all(corr[u] == 1.f);
     }
-    if (!__all(corr == 1.f)) {
+    if (rescale) {
 #pragma unroll
-      for (int dt = 0; dt < DT; ++dt) o[dt] *= corr;
+      for (int u = 0; u < NSUB; ++u)
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) o[u][dt] *= corr[u];
     }
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
       for (int kk = 0; kk < 2; ++kk) {
         const bf16x8 a = *reinterpret_cast<const bf16x8*>(vimg + (16 * dt + c16) * PV + 16 * (4 * kk + g));
-        o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pf[kk], o[dt], 0, 0, 0);
+#pragma unroll
+        for (int u = 0; u < NSUB; ++u) o[u][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pf[u][kk], o[u][dt], 0, 0, 0);
       }
   }
-  if (!valid) return;
-  if (splits == 1) {
-    const float inv = l > 0.f ? 1.f / l : 0.f;
-    float* dst = out + (row * heads + head) * vall_total + (long)chunk * VALL + 4 * g;
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt) *reinterpret_cast<f32x4*>(dst + 16 * dt) = o[dt] * inv;
-  } else {
-    const long rec = (row * heads + head) * splits + blockIdx.z;
-    float* dst = ws_o + rec * vall_total + (long)chunk * VALL + 4 * g;
+  for (int u = 0; u < NSUB; ++u) {
+    if (!valid[u]) continue;
+    if (splits == 1) {
+      const float inv = l[u] > 0.f ? 1.f / l[u] : 0.f;
+      float* dst = out + (row[u] * heads + head[u]) * vall_total + (long)chunk * VALL + 4 * g;
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt) *reinterpret_cast<f32x4*>(dst + 16 * dt) = o[dt];
-    if (g == 0 && chunk == 0) {
-      ws_ml[2 * rec] = m;
-      ws_ml[2 * rec + 1] = l;
+      for (int dt = 0; dt < DT; ++dt) *reinterpret_cast<f32x4*>(dst + 16 * dt) = o[u][dt] * inv;
+    } else {
+      const long rec = (row[u] * heads + head[u]) * splits + blockIdx.z;
+      float* dst = ws_o + rec * vall_total + (long)chunk * VALL + 4 * g;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) *reinterpret_cast<f32x4*>(dst + 16 * dt) = o[u][dt];
+      if (g == 0 && chunk == 0) {
+        ws_ml[2 * rec] = m[u];
+        ws_ml[2 * rec + 1] = l[u];
+      }
     }
   }
 }
@@ -931,7 +958,12 @@ VPSA_EXPORT int vpsa_window_mfma_supported(int heads, int kv_heads, int dim, int
          heads / kv_heads <= 64;
 }
 
-template <int DIM, int VALL>
+// Runs of 16 slots per wave in prefill tiles.  Two (a tile of 128 slots, every LDS fragment read half as often per
+// slot) need 256 accumulator registers per lane at 512 value channels; the compiler keeps them in the 256 arch
+// registers and spills (1.4 ms against 0.6 ms per 8192 rows), so one it is until the accumulators are placed by hand.
+#define WINDOW_PREFILL_SUB 1
+
+template <int DIM, int VALL, int NSUB>
 static int launch_window_mfma(const void* q, long q_stride, const void* cache, long page_stride, const int* block_tables,
                               int bt_stride, const int* tiles, const int* positions, const float* sink, float* out,
                               int n_tiles, int heads, int kv_heads, int window, int keep_first, float scale,
@@ -939,18 +971,21 @@ static int launch_window_mfma(const void* q, long q_stride, const void* cache, l
   constexpr int LDS = PAGE * (DIM * 2 + 16) + VALL * (PAGE * 2 + 16);
   static bool attr_set = false;
   if (!attr_set) {
-    if (hipFuncSetAttribute((const void*)window_mfma_kernel<DIM, VALL>, hipFuncAttributeMaxDynamicSharedMemorySize,
+    if (hipFuncSetAttribute((const void*)window_mfma_kernel<DIM, VALL, NSUB>, hipFuncAttributeMaxDynamicSharedMemorySize,
                             LDS) != hipSuccess)
       return -2;
     attr_set = true;
   }
-  window_mfma_kernel<DIM, VALL><<<dim3(n_tiles, kv_heads * n_chunks, splits), dim3(256), LDS, st>>>(
+  window_mfma_kernel<DIM, VALL, NSUB><<<dim3(n_tiles, kv_heads * n_chunks, splits), dim3(256), LDS, st>>>(
       (const uint16_t*)q, q_stride, (const uint16_t*)cache, page_stride, block_tables, bt_stride, tiles, positions, sink,
       out, heads, kv_heads, window, keep_first, scale, softcap, splits, ws_o, ws_ml, n_chunks);
   if (splits > 1)  // decode rows only: row r of the launch is row r of out
     window_merge_kernel<<<n_tiles * heads, 128, 0, st>>>(ws_o, ws_ml, sink, out, heads, VALL * n_chunks, splits);
   return 0;
 }
+
+// (row, query head) pairs of one prefill tile of the matrix-core kernel
+VPSA_EXPORT int vpsa_window_tile_slots() { return 64 * WINDOW_PREFILL_SUB; }
 
 // tiles: int32 [n_tiles][4] = (sequence, first row, rows, position of the first row), -1 sequence = skip;
 // nullptr: n_tiles decode rows, row r = sequence r at positions[r].
@@ -964,10 +999,16 @@ VPSA_EXPORT int vpsa_window_attention_mfma(const void* q, long q_stride, const v
   if (splits < 1 || (splits > 1 && (tiles || !ws_o || !ws_ml))) return 3;  // splits are for decode rows
   const int vall = window_chunk(kv_heads * vdim), n_chunks = kv_heads * vdim / vall;
 #define WM(D, V)                                                                                                      \
-  if (dim == D && vall == V)                                                                                          \
-    return launch_window_mfma<D, V>(q, q_stride, cache, page_stride, block_tables, bt_stride, tiles, positions, sink,  \
-                                    out, n_tiles, heads, kv_heads, window, keep_first, scale, softcap, splits, ws_o,     \
-                                    ws_ml, n_chunks, stream);
+  if (dim == D && vall == V) {                                                                                        \
+    if (tiles)                                                                                                        \
+      return launch_window_mfma<D, V, WINDOW_PREFILL_SUB>(q, q_stride, cache, page_stride, block_tables, bt_stride,    \
+                                                          tiles, positions, sink, out, n_tiles, heads, kv_heads,      \
+                                                          window, keep_first, scale, softcap, splits, ws_o, ws_ml,     \
+                                                          n_chunks, stream);                                          \
+    return launch_window_mfma<D, V, 1>(q, q_stride, cache, page_stride, block_tables, bt_stride, tiles, positions,     \
+                                       sink, out, n_tiles, heads, kv_heads, window, keep_first, scale, softcap,       \
+                                       splits, ws_o, ws_ml, n_chunks, stream);                                        \
+  }
   WM(64, 128) WM(64, 256) WM(64, 512) WM(128, 128) WM(128, 256) WM(128, 512)
 #undef WM
   return 2;

@@ -42,7 +42,7 @@ def _kernels():
             "vpsa_gather_rows", "vpsa_moe_finish", "vpsa_latent_mfma_supported", "vpsa_latent_attention_mfma",
             "vpsa_moe_mfma_act",
             "vpsa_add_dyt", "vpsa_recurrent_scan", "vpsa_head_rms", "vpsa_short_conv_qkv", "vpsa_window_attention",
-            "vpsa_mix_heads", "vpsa_xielu", "vpsa_window_mfma_supported", "vpsa_window_attention_mfma",
+            "vpsa_mix_heads", "vpsa_xielu", "vpsa_window_mfma_supported", "vpsa_window_attention_mfma", "vpsa_window_tile_slots",
         ):
             getattr(lib, name).restype = c_int
         lib.vpsa_prefill_split_record_bytes.restype = c_long

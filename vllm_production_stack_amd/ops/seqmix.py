@@ -222,7 +222,11 @@ def short_conv_qkv(proj, conv_w, heads: int, kv_heads: int, dim: int, vdim: int,
     return q
 
 
-WINDOW_TILE_SLOTS = 64  # (row, query head) pairs of one tile of the matrix-core kernel
+def window_tile_slots() -> int:
+    """(row, query head) pairs of one prefill tile of the matrix-core kernel."""
+    return int(_ops()._kernels().vpsa_window_tile_slots())
+
+
 WINDOW_MFMA = True      # False: every call takes the plain kernel (A/B runs, tests of the plain kernel)
 
 
@@ -233,10 +237,10 @@ def window_mfma_supported(heads: int, kv_heads: int, dim: int, vdim: int) -> boo
 def build_window_tiles(q_lens, ctx_lens, heads: int, kv_heads: int):
     """Work list of the matrix-core kernel for the prefill part of a batch: int32 rows (sequence, first
     query row, rows, position of the first row); a tile holds consecutive rows of one sequence, as many as
-    fit 64 (row, query head of one KV group) pairs.  Latest rows first (they visit the most pages)."""
+    fit the kernel's slots ((row, query head of one KV group) pairs).  Latest rows first (they visit the most pages)."""
     import numpy as np
 
-    per = max(1, WINDOW_TILE_SLOTS // (heads // kv_heads))
+    per = max(1, window_tile_slots() // (heads // kv_heads))
     parts = []
     row = 0
     for i, (n, ctx) in enumerate(zip(q_lens, ctx_lens)):
