@@ -141,7 +141,7 @@ __global__ __launch_bounds__(256) void scan_prepare_kernel(const T* __restrict__
 //          scan_propagate_kernel then walks a sequence's pieces, S <- A_piece (.) S + end state, leaves every
 //          piece's START state in ws_state and the sequence's end state in its slot;
 // PHASE 2: a piece's outputs from its start state.
-template <typename T, int RPT, bool GATED, int PHASE>
+template <typename T, int RPT, bool GATED, bool FOLD, int PHASE>
 __global__ __launch_bounds__(256) void recurrent_scan_kernel(
     const T* __restrict__ proj, long p_stride, int v_col, int heads, int dim, int vdim, const float* __restrict__ prep,
     float* __restrict__ state, long state_stride, const int* __restrict__ seq_cu, const int* __restrict__ seq_state,
@@ -195,6 +195,11 @@ __global__ __launch_bounds__(256) void recurrent_scan_kernel(
     }
   }
   const float dec = GATED ? 0.f : decay[head];
+  // A fixed decay is folded into the staged block: with S~_t = S_t / dec^(t+1) inside a block of TB tokens the
+  // update is one multiply-add, S~_t = S~_(t-1) + (k_t / dec^(t+1)) v_t^T, the read-out another,
+  // o_t = S~_t^T (dec^(t+1) q_t), and the block ends with S = S~ dec^nb.  (Two operations per state element and
+  // token instead of three.)  Decays whose TB-th power leaves fp32's comfortable range take the plain form (FOLD off).
+  constexpr bool folded = FOLD && !GATED;  // the caller checks the decays (dec^TB well inside fp32's range)
   if (dimp > dim)  // rows past the head's size stay zero in every staged block
     for (int e = tid; e < TB * NP * dimp; e += 256) smem[e] = 0.f;
   for (int rb = r0; rb < r1; rb += TB) {
@@ -204,7 +209,12 @@ __global__ __launch_bounds__(256) void recurrent_scan_kernel(
       const int tt = e / (NP * dim), rem = e - tt * (NP * dim);
       const int which = rem / dim, i = rem - which * dim;
       if (PHASE == 1 && which == 0) continue;         // no outputs: no queries
-      const float x = prep[((long)(rb + tt) * heads + head) * NP * dim + rem];
+      float x = prep[((long)(rb + tt) * heads + head) * NP * dim + rem];
+      if (folded) {
+        float pw = dec;
+        for (int t = 0; t < tt; ++t) pw *= dec;       // dec^(tt + 1)
+        x = which == 0 ? x * pw : x / pw;
+      }
       (which == 0 ? qs : which == 1 ? ks : as)[tt * dimp + i] = x;
     }
     for (int e = tid; e < nb * cols; e += 256) {
@@ -230,12 +240,22 @@ __global__ __launch_bounds__(256) void recurrent_scan_kernel(
           const int j = jg * 4 + jj;
 #pragma unroll
           for (int c = 0; c < 4; ++c) {
-            S[j][c] = fmaf(a4[jj], S[j][c], k4[jj] * v[c]);
+            S[j][c] = folded ? fmaf(k4[jj], v[c], S[j][c]) : fmaf(a4[jj], S[j][c], k4[jj] * v[c]);
             if (PHASE != 1) acc[c] = fmaf(S[j][c], q4[jj], acc[c]);
           }
         }
       }
+      if (folded && tt == nb - 1) {  // back to the true state at the block's end
+        float pw = 1.f;
+        for (int t = 0; t < nb; ++t) pw *= dec;
+#pragma unroll
+        for (int j = 0; j < RPT; ++j)
+#pragma unroll
+          for (int c = 0; c < 4; ++c) S[j][c] *= pw;
+      }
       if (PHASE != 1) {
+        // (DPP adds instead of these shuffles were measured: 1.31 -> 1.46 ms per 8192 rows, their wait states sit
+        // on the chain from the last multiply-add to the store)
         for (int off = R >> 1; off > 0; off >>= 1) {
 #pragma unroll
           for (int c = 0; c < 4; ++c) acc[c] += __shfl_xor(acc[c], off, 64);
@@ -843,14 +863,15 @@ static void scan_shape(int dim, int* rpt, int* r) {
 // pieces: nullptr = every sequence in one go (its rows from seq_cu); else int32 [n_pieces][3] = (sequence, first row,
 // rows) in sequence order, seq_pieces int32 [n_seqs + 1] = a sequence's first piece, and the workspaces
 // ws_state fp32 [n_pieces, heads, dim, vdim], ws_decay fp32 [n_pieces, heads, dim].  prep: fp32 workspace
-// [rows, heads, 2 (3 when gated), dim].
+// [rows, heads, 2 (3 when gated), dim].  fold: every decay's 16th power is well inside fp32's range (the kernel
+// then folds the decay into the staged keys and queries).
 VPSA_EXPORT int vpsa_recurrent_scan(const void* proj, long p_stride, int q_col, int k_col, int v_col, int heads, int dim,
                                     int vdim, float* state, long state_stride, const int* seq_cu, const int* seq_state,
                                     int n_seqs, const int* positions, const float* decay, const float* cos_sin,
                                     int rot_dims, int layout, float k_scale, const float* gate_bias,
                                     const float* gate_lower, float* out, int gated, const int* pieces,
                                     const int* seq_pieces, int n_pieces, float* ws_state, float* ws_decay, float* prep,
-                                    int rows, int dt, hipStream_t stream) {
+                                    int rows, int fold, int dt, hipStream_t stream) {
   if (n_seqs <= 0 || rows <= 0) return 0;
   int rpt, r;
   scan_shape(dim, &rpt, &r);
@@ -862,17 +883,18 @@ VPSA_EXPORT int vpsa_recurrent_scan(const void* proj, long p_stride, int q_col, 
   if (tb < 1) return 3;
   const size_t lds = (size_t)tb * per_tok * sizeof(float);
   const int col_blocks = (vdim + cols - 1) / cols;
-#define SCAN(RPT, G, PH, NZ)                                                                                           \
-  recurrent_scan_kernel<T, RPT, G, PH><<<dim3(col_blocks, heads, NZ), 256, lds, stream>>>(                             \
+#define SCAN(RPT, G, F, PH, NZ)                                                                                        \
+  recurrent_scan_kernel<T, RPT, G, F, PH><<<dim3(col_blocks, heads, NZ), 256, lds, stream>>>(                          \
       (const T*)proj, p_stride, v_col, heads, dim, vdim, prep, state, state_stride, seq_cu, seq_state, positions,     \
       decay, out, r, tb, pieces, ws_state)
-#define SCAN_R(G, PH, NZ)                          \
-  if (rpt == 8) SCAN(8, G, PH, NZ);                \
-  else if (rpt == 16) SCAN(16, G, PH, NZ);         \
-  else SCAN(32, G, PH, NZ);
+#define SCAN_R(G, F, PH, NZ)                       \
+  if (rpt == 8) SCAN(8, G, F, PH, NZ);             \
+  else if (rpt == 16) SCAN(16, G, F, PH, NZ);      \
+  else SCAN(32, G, F, PH, NZ);
 #define SCAN_G(PH, NZ)                             \
-  if (gated) { SCAN_R(true, PH, NZ) }              \
-  else { SCAN_R(false, PH, NZ) }
+  if (gated) { SCAN_R(true, false, PH, NZ) }       \
+  else if (fold) { SCAN_R(false, true, PH, NZ) }   \
+  else { SCAN_R(false, false, PH, NZ) }
   if (gated) {
     SM_DISPATCH(dt, (scan_prepare_kernel<T, true><<<rows, 256, 0, stream>>>((const T*)proj, p_stride, q_col, k_col, heads,
                                                                             dim, positions, cos_sin, rot_dims, layout,

@@ -153,6 +153,8 @@ def case_recurrences(dev, dtype, tol):
         n_state = heads * dim * vdim
         for want, kw in ((want_decay, dict(decay=decay.to(dev), cos_sin=table.to(dev), rot_dims=rot_dims, layout=layout,
                                            k_scale=0.25)),
+                         (want_decay, dict(decay=decay.to(dev), cos_sin=table.to(dev), rot_dims=rot_dims, layout=layout,
+                                           k_scale=0.25, min_decay=float(decay.min()))),  # decay folded into the block
                          (want_gate, dict(gate_bias=bias.to(dev), gate_lower=lower.to(dev)))):
             state = torch.full((3, n_state + 7), float("nan"), device=dev)  # a chunk at position 0 must not read it
             pd = proj.to(dev)
@@ -200,6 +202,7 @@ def case_recurrence_pieces(dev, dtype, tol):
         assert cut is not None and cut[0].shape[0] > 5
         pieces = tuple(torch.from_numpy(a).to(dev) for a in cut)
         for kw in (dict(decay=decay, cos_sin=table, rot_dims=dim, layout=0, k_scale=dim ** -0.5),
+                   dict(decay=decay, cos_sin=table, rot_dims=dim, layout=0, k_scale=dim ** -0.5, min_decay=float(decay.min())),
                    dict(gate_bias=bias, gate_lower=lower)):
             s0 = torch.randn(3, heads * dim * vdim + 4, generator=g).to(dev)
             res = []

@@ -239,7 +239,8 @@ class RevelixModel:
         proj = ops.linear(h, lw.w_in)  # q | k | v | g
         o = ops.recurrent_scan(proj, 0, hd, 2 * hd, m.heads, m.dim, m.vdim, self.state, lw.state_off, meta.seq_cu,
                                meta.seq_state, meta.positions, decay=lw.decay, cos_sin=lw.cos_sin, rot_dims=m.rot.dims,
-                               layout=LAYOUTS[m.rot.layout], k_scale=m.dim ** -0.5, pieces=meta.scan_pieces)
+                               layout=LAYOUTS[m.rot.layout], k_scale=m.dim ** -0.5, pieces=meta.scan_pieces,
+                               min_decay=min(m.decay))
         y = ops.head_rms_norm(o, self.cfg.norm_eps, self.dtype, gate=proj[:, 2 * hd + hv:2 * hd + 2 * hv])
         return ops.linear(y, lw.w_o)
 

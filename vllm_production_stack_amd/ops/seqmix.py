@@ -94,6 +94,7 @@ def add_dyt_norm(residual, deltas, weight, bias, alpha, out_dtype, want_out: boo
     return y
 
 
+SCAN_FOLD_MIN_DECAY = 0.1    # decay^-16 stays below 1e16
 SCAN_PIECE_MIN_ROWS = 128   # sequences of a step shorter than this are walked in one go
 SCAN_PIECES_TARGET = 96     # pieces per launch that fill the chip (times heads and column blocks)
 
@@ -119,7 +120,7 @@ def build_scan_pieces(q_lens, target: int = SCAN_PIECES_TARGET):
 
 def recurrent_scan(proj, q_col: int, k_col: int, v_col: int, heads: int, dim: int, vdim: int, state, state_off: int,
                    seq_cu, seq_state, positions, *, decay=None, cos_sin=None, rot_dims: int = 0, layout: int = 0,
-                   k_scale: float = 1.0, gate_bias=None, gate_lower=None, pieces=None):
+                   k_scale: float = 1.0, gate_bias=None, gate_lower=None, pieces=None, min_decay: float = 0.0):
     """Per sequence and head, over the sequence's rows in order: S <- a_t (.) S + k_t v_t^T, o_t = S^T q_t
     with S [dim, vdim] carried in the sequence's state slot.  q, k and v are column ranges of ``proj``
     [T, cols] (heads side by side).
@@ -127,6 +128,10 @@ def recurrent_scan(proj, q_col: int, k_col: int, v_col: int, heads: int, dim: in
     ``decay`` (fp32 [heads]): a_t = decay[head] for every row of S; q and k turn by the rotary table
     ``cos_sin`` over their first ``rot_dims`` channels (``layout`` 0: pairs (i, i + rot_dims / 2), 1: pairs
     (2 i, 2 i + 1)) and k is multiplied by ``k_scale`` afterwards.
+
+    ``min_decay``: the smallest of the decays as the host knows it; from ``SCAN_FOLD_MIN_DECAY`` up the kernel
+    folds the decay into the staged keys and queries of a 16-token block (two operations per state element and
+    token instead of three).
 
     ``gate_bias`` / ``gate_lower`` (fp32 [heads * dim]) instead: the k columns hold gate logits,
     a_t = lower + (1 - lower) sigmoid(logit + bias) per row of S, k_t = 1 - a_t, q = silu(q).
@@ -165,7 +170,8 @@ def recurrent_scan(proj, q_col: int, k_col: int, v_col: int, heads: int, dim: in
         c_int(vdim), _at(state, state_off), c_long(state.stride(0)), o._p(seq_cu), o._p(seq_state),
         c_int(seq_state.numel()), o._p(positions), o._p(decay), o._p(cos_sin), c_int(rot_dims), c_int(layout),
         c_float(k_scale), o._p(gate_bias), o._p(gate_lower), o._p(out), c_int(1 if gated else 0), o._p(pc), o._p(sp),
-        c_int(n_pieces), o._p(ws_state), o._p(ws_decay), o._p(prep), c_int(proj.shape[0]), c_int(_dt(proj)),
+        c_int(n_pieces), o._p(ws_state), o._p(ws_decay), o._p(prep), c_int(proj.shape[0]),
+        c_int(1 if (not gated and min_decay >= SCAN_FOLD_MIN_DECAY) else 0), c_int(_dt(proj)),
         o._stream()), "recurrent_scan")
     return out
 
