@@ -136,3 +136,18 @@ def test_decode_graphs_match_eager(dtype, model_a):
     assert outs[True] == outs[False]
     if dtype == "float32":
         assert outs[True][0] == ro.greedy(cfg, w, prompts[0], 24)
+
+
+def test_sleep_and_wake_keep_the_tokens(model_a):
+    """The state pool leaves with the KV pool and comes back; stochastic sampling takes the fp32 logits."""
+    cfg, w = model_a
+    eng = rc.make_engine(cfg, w, "cuda", "bfloat16", pages=8, slots=3, eager=False)
+    prompts = [rc.tokens(cfg, n, 200 + n) for n in (50, 3, 70)]
+    greedy = SamplingParams(max_tokens=12, temperature=0.0, ignore_eos=True)
+    first = eng.generate(prompts, greedy)
+    sampled = eng.generate(prompts[:2], SamplingParams(max_tokens=8, temperature=0.9, top_p=0.9, seed=3, ignore_eos=True))
+    assert [len(o) for o in sampled] == [8, 8]
+    assert eng.sleep(1) > 0 and eng.runner.state_pool is None
+    eng.wake_up()
+    assert eng.generate(prompts, greedy) == first
+    eng.shutdown()

@@ -484,6 +484,37 @@ PRESETS["zururax-bench"] = zururax_config(
      for i in range(8)],
     max_position_embeddings=32768)
 
+
+
+def _rx_retention(heads, dim, vdim, mlp=None, base=10000.0):
+    return {"type": "retention", "mlp": mlp,
+            "mixer": {"heads": heads, "dim": dim, "vdim": vdim, "rot": {"base": base, "dims": dim},
+                      "decay": [1 - 2.0 ** (-5 - 3 * i / heads) for i in range(heads)]}}
+
+
+def _rx_parallel(heads, kv_heads, dim, vdim, window, keep, r_heads, r_dim, r_vdim, mlp=None, conv=4):
+    return {"type": "parallel", "mlp": mlp,
+            "mixer": {"left": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "conv": conv,
+                               "mask": {"size": window, "keep_first": keep},
+                               "rot": {"base": 1e6, "dims": dim,
+                                       "scaling": {"factor": 8.0, "original": 4096, "fast": 32.0, "slow": 1.0}},
+                               "scale": dim ** -0.5, "softcap": 50.0},
+                      "right": {"heads": r_heads, "dim": r_dim, "vdim": r_vdim},
+                      "left_scale": 0.7, "right_scale": 0.7}}
+
+
+# Revelix at random weights: a small one for smoke runs, and one with layer shapes of a 2048-wide model
+PRESETS["tiny-revelix"] = revelix_config(
+    "tiny-revelix", 512, 128,
+    [_rx_retention(2, 32, 64, {"kind": "dense", "ff": 256}),
+     _rx_parallel(4, 2, 64, 64, 96, 2, 2, 32, 64, {"kind": "dense", "ff": 256}),
+     _rx_retention(2, 32, 64)], logit_scale=0.5, max_position_embeddings=4096)
+PRESETS["revelix-bench"] = revelix_config(
+    "revelix-bench", 32000, 2048,
+    [_rx_retention(16, 128, 256, {"kind": "dense", "ff": 8192}) if i % 3 == 0 else
+     _rx_parallel(16, 4, 128, 128, 1024, 4, 8, 128, 128, {"kind": "dense", "ff": 8192}) for i in range(6)],
+    logit_scale=0.5, max_position_embeddings=32768)
+
 _ALIASES = {
     "meta-llama/meta-llama-3-8b": "llama-3-8b",
     "meta-llama/meta-llama-3-8b-instruct": "llama-3-8b",

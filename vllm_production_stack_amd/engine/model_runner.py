@@ -77,15 +77,16 @@ class ModelRunner:
         self.page_elems = int(np.prod(self.page_dims))
         self.page_bytes = self.page_elems * torch.empty((), dtype=self.dtype).element_size()
         self.max_pages_per_seq = (self.max_model_len + PAGE - 1) // PAGE
+        # models whose mixers carry state from token to token: one fp32 slot per running sequence, allocated
+        # before the pages are planned from what is left
+        self.stateful = hasattr(self.model, "state_shape")
+        self.state_pool = None
+        self._alloc_state()
         self.num_pages = self._plan_pages()
         self.pool_listeners: list = []  # called with the new pool tensor after a wake-up
         self._pool_dev_ptr = 0       # an allocation of our own behind the pool (exported to peers), or 0
         self.pool_ipc_handle = None  # hex hipIpc handle of that allocation
         self.pool = self._alloc_pool()
-        # models whose mixers carry state from token to token: one fp32 slot per running sequence
-        self.stateful = hasattr(self.model, "state_shape")
-        self.state_pool = None
-        self._alloc_state()
         self.sampler = Sampler(device, cfg.seed)
         # graphs need the HIP attention kernels (the generic path reads lengths on the host)
         self.use_graphs = (device.type == "cuda" and not cfg.enforce_eager
