@@ -72,10 +72,10 @@ def config_d():
 
 
 def config_e():
-    """Parallel layers only; a window of one position; two taps."""
+    """Parallel layers only; a window of one position; two and five taps; a value size that is no multiple of 4."""
     return ro.make_config([ro.parallel_layer(heads=2, kv_heads=2, dim=8, vdim=12, conv=2, size=1, keep=2, r_heads=1, r_dim=4,
                                              r_vdim=6),
-                           ro.parallel_layer(heads=2, kv_heads=1, dim=16, vdim=8, conv=5, size=200, keep=0, rot_dims=4,
+                           ro.parallel_layer(heads=2, kv_heads=1, dim=16, vdim=6, conv=5, size=200, keep=0, rot_dims=4,
                                              r_heads=2, r_dim=8, r_vdim=4, mlp={"kind": "dense", "ff": 16})],
                           vocab=40, width=16, logit_scale=0.25)
 
